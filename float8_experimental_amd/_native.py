@@ -1,0 +1,282 @@
+"""ctypes binding of ``libf8mi.so`` (the C ABI declared in ``include/f8mi.h``).
+
+Torch is used here for device memory and streams only: every function takes
+torch tensors, checks them on the host, and hands raw device pointers plus the
+current HIP stream to the library.  There is no fallback: if the library is
+missing, cannot be loaded, or the tensors are not on a GPU, the call raises.
+"""
+import ctypes as C
+import os
+import threading
+from typing import Optional, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libf8mi.so")
+
+BF16, FP16, FP32 = 0, 1, 2
+E4M3FN, E5M2 = 0, 1
+K_AMAX, K_CAST, K_GEMM, K_SYNC = 0, 1, 2, 3
+
+_DT = {torch.bfloat16: BF16, torch.float16: FP16, torch.float32: FP32}
+_F8 = {torch.float8_e4m3fn: E4M3FN, torch.float8_e5m2: E5M2}
+
+EXPORTS = (
+    "f8mi_version",
+    "f8mi_last_error",
+    "f8mi_device_info",
+    "f8mi_workspace_bytes",
+    "f8mi_amax_scale",
+    "f8mi_cast",
+    "f8mi_gemm_nt",
+    "f8mi_sync",
+    "f8mi_delayed_init",
+    "f8mi_prof_enable",
+    "f8mi_prof_reset",
+    "f8mi_prof_read",
+)
+
+_lib = None
+_lock = threading.Lock()
+
+
+class Float8NativeError(RuntimeError):
+    pass
+
+
+def lib() -> C.CDLL:
+    """Loads libf8mi.so once.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise Float8NativeError(
+                f"{LIB_PATH} not found: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(or `python float8_experimental_amd/_build.py`); there is no fallback path"
+            )
+        L = C.CDLL(LIB_PATH)
+        vp, i64, i32, fp = C.c_void_p, C.c_int64, C.c_int, C.c_void_p
+        L.f8mi_version.restype = i32
+        L.f8mi_version.argtypes = []
+        L.f8mi_last_error.restype = C.c_char_p
+        L.f8mi_last_error.argtypes = []
+        L.f8mi_device_info.restype = i32
+        L.f8mi_device_info.argtypes = [i32, C.POINTER(i32), C.POINTER(i32), C.c_char_p, i32]
+        L.f8mi_workspace_bytes.restype = C.c_size_t
+        L.f8mi_workspace_bytes.argtypes = []
+        L.f8mi_amax_scale.restype = i32
+        L.f8mi_amax_scale.argtypes = [vp, i64, i64, i64, i32, i32, i32, i32, fp, fp, vp, vp]
+        L.f8mi_cast.restype = i32
+        L.f8mi_cast.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, vp, fp, vp, vp]
+        L.f8mi_gemm_nt.restype = i32
+        L.f8mi_gemm_nt.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
+        L.f8mi_sync.restype = i32
+        L.f8mi_sync.argtypes = [vp, i32, i32, i32, i32, vp]
+        L.f8mi_delayed_init.restype = i32
+        L.f8mi_delayed_init.argtypes = [fp, fp, fp, i32, i32, i32, vp]
+        L.f8mi_prof_enable.restype = i32
+        L.f8mi_prof_enable.argtypes = [i32]
+        L.f8mi_prof_reset.restype = i32
+        L.f8mi_prof_reset.argtypes = []
+        L.f8mi_prof_read.restype = i32
+        L.f8mi_prof_read.argtypes = [i32, C.POINTER(C.c_uint64), C.POINTER(C.c_double), C.POINTER(C.c_double)]
+        _lib = L
+    return _lib
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().f8mi_last_error().decode(errors="replace")
+        raise Float8NativeError(f"{what} failed with code {rc}: {msg}")
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise Float8NativeError(
+            f"{name} is on {t.device}: float8_experimental_amd computes on MI355X device tensors only "
+            "(no CPU fallback)"
+        )
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+_checked_devices = set()
+
+
+def _check_device(dev: torch.device) -> None:
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    if idx in _checked_devices:
+        return
+    arch = C.create_string_buffer(64)
+    cu, lds = C.c_int(0), C.c_int(0)
+    _check(lib().f8mi_device_info(idx, C.byref(cu), C.byref(lds), arch, 64), "f8mi_device_info")
+    _checked_devices.add(idx)
+
+
+_workspaces = {}
+
+
+def workspace(dev: torch.device) -> torch.Tensor:
+    """Zero-filled reduction workspace, one per (device, stream); kernels re-zero it themselves."""
+    _check_device(dev)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(lib().f8mi_workspace_bytes() // 4, dtype=torch.int32, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
+def _as_2d(x: torch.Tensor) -> Tuple[torch.Tensor, int, int, int]:
+    """(tensor whose memory is read, rows, cols, row stride) -- copies only when the layout needs it."""
+    if x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= x.shape[1] and x.shape[0] > 0 and x.shape[1] > 0:
+        return x, x.shape[0], x.shape[1], x.stride(0)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    cols = x.shape[-1] if x.dim() > 0 else 1
+    rows = x.numel() // cols if cols else 0
+    return x, rows, cols, cols
+
+
+def amax_scale(x: torch.Tensor, float8_dtype: torch.dtype, math_dtype: Optional[torch.dtype] = None,
+               orig_is_fp16: Optional[bool] = None, want_amax: bool = True, want_scale: bool = True,
+               amax_out: Optional[torch.Tensor] = None, scale_out: Optional[torch.Tensor] = None):
+    """max|x| (fp32, 0-dim) and its fp8 scale (fp32, 0-dim) in one pass.  See f8mi_amax_scale."""
+    _require_gpu(x, "x")
+    xs, rows, cols, ld = _as_2d(x)
+    if math_dtype is None:
+        math_dtype = x.dtype
+    if orig_is_fp16 is None:
+        orig_is_fp16 = x.dtype == torch.float16
+    amax = amax_out if amax_out is not None else (torch.empty((), dtype=torch.float32, device=x.device) if want_amax else None)
+    scale = scale_out if scale_out is not None else (torch.empty((), dtype=torch.float32, device=x.device) if want_scale else None)
+    for o in (amax, scale):
+        if o is not None:
+            assert o.dtype == torch.float32 and o.numel() == 1 and o.device == x.device
+    ws = workspace(x.device)
+    rc = lib().f8mi_amax_scale(xs.data_ptr(), rows, cols, ld, _DT[x.dtype], _F8[float8_dtype], _DT[math_dtype],
+                               int(orig_is_fp16), amax.data_ptr() if amax is not None else None,
+                               scale.data_ptr() if scale is not None else None, ws.data_ptr(), _stream(x))
+    _check(rc, "f8mi_amax_scale")
+    return amax, scale
+
+
+def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, product_dtype: Optional[torch.dtype] = None,
+         want_out: bool = True, want_out_t: bool = False, amax_out: Optional[torch.Tensor] = None):
+    """Saturated fp8 cast of a tensor viewed as [rows, cols=last dim].
+
+    Returns (out, out_t): ``out`` has x's shape; ``out_t`` is the dense [cols, rows]
+    transpose of the flattened 2-D view.  ``amax_out`` (fp32, 1 element), if given,
+    receives max|x| computed in the same pass.  See f8mi_cast.
+    """
+    _require_gpu(x, "x")
+    assert scale.dtype == torch.float32 and scale.numel() == 1 and scale.device == x.device, "scale: 1 fp32 element on x's device"
+    xs, rows, cols, ld = _as_2d(x)
+    if product_dtype is None:
+        product_dtype = x.dtype
+    out = torch.empty(x.shape, dtype=float8_dtype, device=x.device) if want_out else None
+    out_t = torch.empty((cols, rows), dtype=float8_dtype, device=x.device) if want_out_t else None
+    ws = None
+    if amax_out is not None:
+        assert amax_out.dtype == torch.float32 and amax_out.numel() == 1 and amax_out.device == x.device
+        ws = workspace(x.device)
+    else:
+        _check_device(x.device)
+    rc = lib().f8mi_cast(xs.data_ptr(), rows, cols, ld, _DT[x.dtype], scale.data_ptr(), _DT[product_dtype],
+                         _F8[float8_dtype], out.data_ptr() if out is not None else None,
+                         out_t.data_ptr() if out_t is not None else None,
+                         amax_out.data_ptr() if amax_out is not None else None,
+                         ws.data_ptr() if ws is not None else None, _stream(x))
+    _check(rc, "f8mi_cast")
+    return out, out_t
+
+
+def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: torch.Tensor, out_dtype: torch.dtype,
+            bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[m, n] = (a[m, :] . bt[n, :]) / (a_scale * b_scale) (+ bias[n]).
+
+    ``a`` is fp8 [m, k], ``bt`` is fp8 [n, k]; both must have unit stride along k.
+    See f8mi_gemm_nt.
+    """
+    _require_gpu(a, "a")
+    _require_gpu(bt, "bt")
+    assert a.dim() == 2 and bt.dim() == 2 and a.shape[1] == bt.shape[1], f"shape mismatch {tuple(a.shape)} x {tuple(bt.shape)}^T"
+    assert a.dtype in _F8 and bt.dtype in _F8, "operands must be float8_e4m3fn / float8_e5m2"
+    m, k = a.shape
+    n = bt.shape[0]
+
+    def rowmajor(t):
+        if t.shape[1] <= 1 or t.stride(1) == 1:
+            if t.shape[0] <= 1 or t.stride(0) >= max(t.shape[1], 1):
+                return t, (t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1))
+        t = t.contiguous()
+        return t, max(t.shape[1], 1)
+
+    a, lda = rowmajor(a)
+    bt, ldb = rowmajor(bt)
+    lda, ldb = max(lda, k), max(ldb, k)
+    for s in (a_scale, b_scale):
+        assert s.dtype == torch.float32 and s.numel() == 1 and s.device == a.device, "scales: 1 fp32 element on the operands' device"
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    else:
+        assert out.shape == (m, n) and out.dtype == out_dtype and out.is_contiguous()
+    if bias is not None:
+        assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a.device
+    _check_device(a.device)
+    rc = lib().f8mi_gemm_nt(a.data_ptr(), _F8[a.dtype], lda, bt.data_ptr(), _F8[bt.dtype], ldb, m, n, k,
+                            a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
+                            bias.data_ptr() if bias is not None else None, _stream(a))
+    _check(rc, "f8mi_gemm_nt")
+    return out
+
+
+def sync_table(entries, device: torch.device) -> torch.Tensor:
+    """Device pointer table for f8mi_sync.  entries: iterable of (amax, history, scale, float8_dtype)."""
+    rows = []
+    for amax, hist, scale, f8 in entries:
+        for t in (amax, hist, scale):
+            _require_gpu(t, "buffer")
+            assert t.dtype == torch.float32 and t.is_contiguous()
+        rows.append([amax.data_ptr(), hist.data_ptr(), scale.data_ptr(), _F8[f8]])
+    return torch.tensor(rows, dtype=torch.int64, device="cpu").to(device)
+
+
+def sync(table: torch.Tensor, hist_len: int, orig_is_fp16: bool, writeback_history: bool = False) -> None:
+    _require_gpu(table, "table")
+    assert table.dtype == torch.int64 and table.dim() == 2 and table.shape[1] == 4 and table.is_contiguous()
+    _check_device(table.device)
+    rc = lib().f8mi_sync(table.data_ptr(), table.shape[0], hist_len, int(orig_is_fp16), int(writeback_history),
+                         _stream(table))
+    _check(rc, "f8mi_sync")
+
+
+def delayed_init(amax: torch.Tensor, history: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype,
+                 orig_is_fp16: bool) -> None:
+    for t in (amax, history, scale):
+        _require_gpu(t, "buffer")
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    _check_device(amax.device)
+    rc = lib().f8mi_delayed_init(amax.data_ptr(), history.data_ptr(), scale.data_ptr(), history.numel(),
+                                 _F8[float8_dtype], int(orig_is_fp16), _stream(amax))
+    _check(rc, "f8mi_delayed_init")
+
+
+def prof_enable(on: bool) -> None:
+    _check(lib().f8mi_prof_enable(int(on)), "f8mi_prof_enable")
+
+
+def prof_reset() -> None:
+    _check(lib().f8mi_prof_reset(), "f8mi_prof_reset")
+
+
+def prof_read(kernel: int):
+    n, ms, work = C.c_uint64(0), C.c_double(0), C.c_double(0)
+    _check(lib().f8mi_prof_read(kernel, C.byref(n), C.byref(ms), C.byref(work)), "f8mi_prof_read")
+    return n.value, ms.value, work.value

@@ -1,0 +1,187 @@
+// K1: max|x| and the fp8 scale in one pass (HBM-bound: reads sizeof(T)*n bytes).
+//
+// |x| is reduced on the raw bit patterns: for IEEE formats the unsigned order
+// of sign-cleared patterns is the order of the magnitudes, and every NaN
+// pattern is larger than inf, so a NaN anywhere wins the max exactly like
+// torch.max propagates it.  Each block folds its result into one word of the
+// workspace with atomicMax; the last block to finish turns the word into
+// amax + scale and zeroes the workspace again.
+#include "f8mi_common.h"
+
+namespace f8mi {
+
+constexpr int AMAX_THREADS = 256;
+constexpr int AMAX_UNROLL = 4;  // 16-byte loads in flight per thread
+
+// sign-cleared patterns of the elements packed in one 32-bit word, reduced to one value
+template <int DT>
+__device__ __forceinline__ uint32_t absmax_word(uint32_t w) {
+    if constexpr (DT == F8MI_FP32) {
+        return w & 0x7fffffffu;
+    } else {
+        uint32_t lo = w & 0x7fffu, hi = (w >> 16) & 0x7fffu;
+        return lo > hi ? lo : hi;
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t absmax_vec(uint4 v, uint32_t m) {
+    uint32_t a = absmax_word<DT>(v.x), b = absmax_word<DT>(v.y);
+    uint32_t c = absmax_word<DT>(v.z), d = absmax_word<DT>(v.w);
+    a = a > b ? a : b;
+    c = c > d ? c : d;
+    a = a > c ? a : c;
+    return m > a ? m : a;
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t absmax_elem(const void* x, int64_t i) {
+    if constexpr (DT == F8MI_FP32) return ((const uint32_t*)x)[i] & 0x7fffffffu;
+    else return (uint32_t)(((const uint16_t*)x)[i] & 0x7fffu);
+}
+
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* lds) {
+    m = wave_max_u32(m);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) lds[wave] = m;
+    __syncthreads();
+    if (wave == 0) {
+        uint32_t v = lane < (int)(blockDim.x >> 6) ? lds[lane] : 0u;
+        m = wave_max_u32(v);
+    }
+    return m;  // valid in wave 0
+}
+
+// Fold this block's max into the workspace; the last block publishes amax/scale.
+__device__ __forceinline__ void publish_amax(uint32_t blockmax, uint32_t* ws, float* amax_out, float* scale_out,
+                                             int in_dt, int math_dt, int fmt, int orig_is_fp16) {
+    if (threadIdx.x == 0) {
+        if (blockmax) atomicMax(&ws[WS_AMAX_BITS], blockmax);
+        __threadfence();
+        uint32_t ticket = atomicAdd(&ws[WS_TICKET], 1u);
+        if (ticket == gridDim.x * gridDim.y - 1) {
+            __threadfence();
+            uint32_t bits = atomicExch(&ws[WS_AMAX_BITS], 0u);
+            atomicExch(&ws[WS_TICKET], 0u);
+            float amax = abs_bits_to_float(bits, in_dt);
+            if (amax_out) *amax_out = amax;
+            if (scale_out) *scale_out = amax_to_scale_dev(amax, math_dt, fmt, orig_is_fp16);
+        }
+    }
+}
+
+// x is dense (ld == cols) and 16-byte aligned: 1-D grid-stride over 16-byte vectors.
+template <int DT>
+__global__ __launch_bounds__(AMAX_THREADS) void amax_dense_kernel(const void* __restrict__ x, int64_t n,
+                                                                   uint32_t* ws, float* amax_out, float* scale_out,
+                                                                   int math_dt, int fmt, int orig_is_fp16) {
+    __shared__ uint32_t red[AMAX_THREADS / 64];
+    constexpr int EPV = DT == F8MI_FP32 ? 4 : 8;
+    const int64_t nvec = n / EPV;
+    const uint4* xv = (const uint4*)x;
+    uint32_t m = 0;
+    const int64_t stride = (int64_t)gridDim.x * AMAX_THREADS;
+    int64_t i = (int64_t)blockIdx.x * AMAX_THREADS + threadIdx.x;
+    for (; i + (AMAX_UNROLL - 1) * stride < nvec; i += AMAX_UNROLL * stride) {
+        uint4 v[AMAX_UNROLL];
+#pragma unroll
+        for (int u = 0; u < AMAX_UNROLL; u++) v[u] = load_nt16(&xv[i + u * stride]);
+#pragma unroll
+        for (int u = 0; u < AMAX_UNROLL; u++) m = absmax_vec<DT>(v[u], m);
+    }
+    for (; i < nvec; i += stride) m = absmax_vec<DT>(load_nt16(&xv[i]), m);
+    if (blockIdx.x == 0) {  // scalar tail (< EPV elements)
+        int64_t t = nvec * EPV + threadIdx.x;
+        if (t < n) {
+            uint32_t a = absmax_elem<DT>(x, t);
+            m = m > a ? m : a;
+        }
+    }
+    m = block_max_u32(m, red);
+    publish_amax(m, ws, amax_out, scale_out, DT, math_dt, fmt, orig_is_fp16);
+}
+
+// Any row stride / alignment: one element per thread step.
+template <int DT>
+__global__ __launch_bounds__(AMAX_THREADS) void amax_strided_kernel(const void* __restrict__ x, int64_t rows,
+                                                                     int64_t cols, int64_t ld, uint32_t* ws,
+                                                                     float* amax_out, float* scale_out, int math_dt,
+                                                                     int fmt, int orig_is_fp16) {
+    __shared__ uint32_t red[AMAX_THREADS / 64];
+    uint32_t m = 0;
+    const int64_t n = rows * cols;
+    const int64_t stride = (int64_t)gridDim.x * AMAX_THREADS;
+    for (int64_t i = (int64_t)blockIdx.x * AMAX_THREADS + threadIdx.x; i < n; i += stride) {
+        int64_t r = i / cols, c = i - r * cols;
+        uint32_t a = absmax_elem<DT>(x, r * ld + c);
+        m = m > a ? m : a;
+    }
+    m = block_max_u32(m, red);
+    publish_amax(m, ws, amax_out, scale_out, DT, math_dt, fmt, orig_is_fp16);
+}
+
+// Empty tensor: torch.max raises; we define amax = 0 so the scale is fmax/eps.
+__global__ void amax_empty_kernel(float* amax_out, float* scale_out, int math_dt, int fmt, int orig_is_fp16) {
+    if (threadIdx.x == 0) {
+        if (amax_out) *amax_out = 0.0f;
+        if (scale_out) *scale_out = amax_to_scale_dev(0.0f, math_dt, fmt, orig_is_fp16);
+    }
+}
+
+static int g_cu_count = 0;
+
+int cu_count() {
+    if (g_cu_count == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            g_cu_count = n;
+        else
+            g_cu_count = 256;
+    }
+    return g_cu_count;
+}
+
+}  // namespace f8mi
+
+using namespace f8mi;
+
+extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt,
+                               int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
+                               void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (rows < 0 || cols < 0 || ld < cols) { set_error("f8mi_amax_scale: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
+    if (in_dtype < 0 || in_dtype > 2 || math_dtype < 0 || math_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_amax_scale: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
+    if (!amax_dev && !scale_dev) { set_error("f8mi_amax_scale: no output requested"); return F8MI_ERR_INVALID_ARG; }
+    const int64_t n = rows * cols;
+    if (n == 0) {
+        hipLaunchKernelGGL(amax_empty_kernel, dim3(1), dim3(64), 0, stream, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        return check_hip(hipGetLastError(), "amax_empty_kernel");
+    }
+    if (!x || !workspace) { set_error("f8mi_amax_scale: null tensor or workspace"); return F8MI_ERR_INVALID_ARG; }
+    uint32_t* ws = (uint32_t*)workspace;
+    const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
+    const bool dense = (ld == cols || rows == 1) && ((uintptr_t)x % 16 == 0);
+    ProfScope prof(F8MI_K_AMAX, (double)n * esz, stream);
+    if (dense) {
+        const int64_t epv = 16 / esz;
+        const int64_t nvec = n / epv;
+        int64_t blocks = (nvec + (int64_t)AMAX_THREADS * AMAX_UNROLL - 1) / ((int64_t)AMAX_THREADS * AMAX_UNROLL);
+        const int64_t cap = (int64_t)cu_count() * 8;
+        if (blocks > cap) blocks = cap;
+        if (blocks < 1) blocks = 1;
+        dim3 g((unsigned)blocks), b(AMAX_THREADS);
+        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_BF16>, g, b, 0, stream, x, n, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP16>, g, b, 0, stream, x, n, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        else hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP32>, g, b, 0, stream, x, n, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+    } else {
+        int64_t blocks = (n + AMAX_THREADS - 1) / AMAX_THREADS;
+        const int64_t cap = (int64_t)cu_count() * 8;
+        if (blocks > cap) blocks = cap;
+        dim3 g((unsigned)blocks), b(AMAX_THREADS);
+        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_strided_kernel<F8MI_BF16>, g, b, 0, stream, x, rows, cols, ld, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP16>, g, b, 0, stream, x, rows, cols, ld, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        else hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP32>, g, b, 0, stream, x, rows, cols, ld, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+    }
+    return check_hip(hipGetLastError(), "amax kernel launch");
+}

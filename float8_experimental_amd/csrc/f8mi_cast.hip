@@ -1,0 +1,286 @@
+// K2 / K2d: saturated fp8 cast, with the transposed copy and (optionally) the
+// tensor's amax fused into the same pass.  HBM-bound: reads sizeof(T) bytes and
+// writes 1 byte per element and per fp8 output.
+//
+// A workgroup of 256 lanes owns a 128 x 128 tile.  Lane t covers columns
+// 8*(t%16) .. +7 of rows 64*h + 4*(t/16) .. +3 for h = 0, 1: eight 16-byte loads
+// (bf16/fp16; sixteen for fp32), all issued before the first use.  The row-major
+// fp8 tile goes out straight from registers as 8-byte stores (16 lanes = one
+// 128-byte row segment).  For the transposed copy each lane transposes its
+// 4 x 8 byte block in registers (v_perm), parks the 4-row dwords in a
+// 128 x 128-byte LDS tile whose dword index is XOR-swizzled by the column group
+// (so the 64 lanes of a store hit 32 banks twice: the floor for 256 bytes), and
+// the tile is read back as 16-byte row pieces: 8 lanes = one 128-byte segment of
+// a row of the transposed output.
+#include "f8mi_common.h"
+
+namespace f8mi {
+
+constexpr int CAST_THREADS = 256;
+constexpr int CAST_TILE = 128;
+
+__device__ __forceinline__ void publish_amax_cast(uint32_t blockmax, uint32_t* ws, float* amax_out, int in_dt) {
+    if (threadIdx.x == 0) {
+        if (blockmax) atomicMax(&ws[WS_AMAX_BITS], blockmax);
+        __threadfence();
+        uint32_t ticket = atomicAdd(&ws[WS_TICKET], 1u);
+        if (ticket == gridDim.x * gridDim.y - 1) {
+            __threadfence();
+            uint32_t bits = atomicExch(&ws[WS_AMAX_BITS], 0u);
+            atomicExch(&ws[WS_TICKET], 0u);
+            *amax_out = abs_bits_to_float(bits, in_dt);
+        }
+    }
+}
+
+// One element: x*scale rounded to PROD, clamped (NaN kept), as fp32 ready for conversion.
+template <int PROD>
+__device__ __forceinline__ float scale_clamp(float x, float scale, float fmax) {
+    float y = round_to<PROD>(__fmul_rn(x, scale));
+    float c = fminf(fmaxf(y, -fmax), fmax);  // drops NaN ...
+    return (y != y) ? y : c;                 // ... so put it back
+}
+
+template <int FMT>
+__device__ __forceinline__ uint32_t pack4(float a, float b, float c, float d) {
+    return cvt2_fp8<FMT>(a, b) | (cvt2_fp8<FMT>(c, d) << 16);
+}
+
+// 4 dwords (rows 0..3, 4 bytes each = columns 0..3) -> 4 dwords (column c: rows 0..3)
+__device__ __forceinline__ void transpose4x4_bytes(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t& c0,
+                                                   uint32_t& c1, uint32_t& c2, uint32_t& c3) {
+    // v_perm_b32(hi, lo, sel): byte i of the result = byte sel[i] of the 8-byte {hi,lo} (lo = bytes 0..3)
+    uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400u);  // r0.b0 r1.b0 r0.b1 r1.b1
+    uint32_t b = __builtin_amdgcn_perm(r1, r0, 0x07030602u);  // r0.b2 r1.b2 r0.b3 r1.b3
+    uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400u);  // r2.b0 r3.b0 r2.b1 r3.b1
+    uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602u);  // r2.b2 r3.b2 r2.b3 r3.b3
+    c0 = __builtin_amdgcn_perm(c, a, 0x05040100u);            // a.b0 a.b1 c.b0 c.b1
+    c1 = __builtin_amdgcn_perm(c, a, 0x07060302u);            // a.b2 a.b3 c.b2 c.b3
+    c2 = __builtin_amdgcn_perm(d, b, 0x05040100u);
+    c3 = __builtin_amdgcn_perm(d, b, 0x07060302u);
+}
+
+template <int DT>
+struct Row8 {  // eight consecutive elements of one row, widened to fp32 on demand
+    uint32_t w[DT == F8MI_FP32 ? 8 : 4];
+};
+
+template <int DT>
+__device__ __forceinline__ float elem(const Row8<DT>& r, int i) {
+    if constexpr (DT == F8MI_FP32) return __uint_as_float(r.w[i]);
+    else {
+        uint32_t h = (i & 1) ? (r.w[i >> 1] >> 16) : (r.w[i >> 1] & 0xffffu);
+        if constexpr (DT == F8MI_BF16) return bf16_bits_to_float(h);
+        else return fp16_bits_to_float(h);
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t absmax_row(const Row8<DT>& r, uint32_t m) {
+    if constexpr (DT == F8MI_FP32) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) { uint32_t a = r.w[i] & 0x7fffffffu; m = m > a ? m : a; }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t lo = r.w[i] & 0x7fffu, hi = (r.w[i] >> 16) & 0x7fffu;
+            m = m > lo ? m : lo;
+            m = m > hi ? m : hi;
+        }
+    }
+    return m;
+}
+
+// Loads 8 elements of row `row` starting at column `col`; out-of-range elements read as +0.
+template <int DT, bool VEC>
+__device__ __forceinline__ void load_row8(Row8<DT>& r, const void* x, int64_t row, int64_t col, int64_t rows,
+                                          int64_t cols, int64_t ld) {
+    constexpr int ESZ = DT == F8MI_FP32 ? 4 : 2;
+    constexpr int NW = DT == F8MI_FP32 ? 8 : 4;
+#pragma unroll
+    for (int i = 0; i < NW; i++) r.w[i] = 0u;
+    if (row >= rows || col >= cols) return;
+    const char* p = (const char*)x + (row * ld + col) * ESZ;
+    if (VEC && col + 8 <= cols) {
+        const uint4* pv = (const uint4*)p;
+        uint4 v0 = load_nt16(pv);
+        r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v0.z; r.w[3] = v0.w;
+        if constexpr (DT == F8MI_FP32) {
+            uint4 v1 = load_nt16(pv + 1);
+            r.w[4] = v1.x; r.w[5] = v1.y; r.w[6] = v1.z; r.w[7] = v1.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (col + i < cols) {
+                if constexpr (DT == F8MI_FP32) r.w[i] = ((const uint32_t*)p)[i];
+                else r.w[i >> 1] |= (uint32_t)((const uint16_t*)p)[i] << ((i & 1) * 16);
+            }
+        }
+    }
+}
+
+template <int DT, int PROD, int FMT, bool VEC>
+__global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
+                                                            int64_t ld, const float* __restrict__ scale_dev,
+                                                            uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
+                                                            float* amax_out, uint32_t* ws) {
+    __shared__ uint32_t tileT[CAST_TILE * CAST_TILE / 4];  // [column][row/4] dwords, swizzled
+    __shared__ uint32_t red[CAST_THREADS / 64];
+
+    const int t = threadIdx.x;
+    const int a = t & 15;   // column group: columns 8a .. 8a+7 of the tile
+    const int b = t >> 4;   // row group: rows 4b .. 4b+3 of each 64-row half
+    const int64_t r0 = (int64_t)blockIdx.y * CAST_TILE;
+    const int64_t c0 = (int64_t)blockIdx.x * CAST_TILE;
+    const int64_t col = c0 + 8 * a;
+
+    Row8<DT> in[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) load_row8<DT, VEC>(in[h][j], x, r0 + 64 * h + 4 * b + j, col, rows, cols, ld);
+
+    const float scale = *scale_dev;
+    constexpr float fmax = FMT == F8MI_E4M3FN ? 448.0f : 57344.0f;
+
+    uint32_t m = 0;
+    if (amax_out) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) m = absmax_row<DT>(in[h][j], m);
+    }
+
+    const bool out_vec = (cols % 8 == 0) && ((uintptr_t)out % 8 == 0);
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float f[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) f[i] = scale_clamp<PROD>(elem<DT>(in[h][j], i), scale, fmax);
+            lo[j] = pack4<FMT>(f[0], f[1], f[2], f[3]);
+            hi[j] = pack4<FMT>(f[4], f[5], f[6], f[7]);
+            const int64_t row = r0 + 64 * h + 4 * b + j;
+            if (out && row < rows && col < cols) {
+                uint8_t* p = out + row * cols + col;
+                if (out_vec) {  // cols % 8 == 0 implies col + 8 <= cols
+                    *(uint2*)p = make_uint2(lo[j], hi[j]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; i++)
+                        if (col + i < cols) p[i] = (uint8_t)((i < 4 ? lo[j] >> (8 * i) : hi[j] >> (8 * (i - 4))) & 0xffu);
+                }
+            }
+        }
+        if (out_t) {
+            uint32_t tc[8];
+            transpose4x4_bytes(lo[0], lo[1], lo[2], lo[3], tc[0], tc[1], tc[2], tc[3]);
+            transpose4x4_bytes(hi[0], hi[1], hi[2], hi[3], tc[4], tc[5], tc[6], tc[7]);
+            const int d = 16 * h + b;              // dword index (rows 4d .. 4d+3) within a tile column
+            const int dsw = d ^ ((a & 7) << 2);    // swizzle by column group
+#pragma unroll
+            for (int cc = 0; cc < 8; cc++) tileT[(8 * a + cc) * (CAST_TILE / 4) + dsw] = tc[cc];
+        }
+    }
+
+    if (out_t) {
+        __syncthreads();
+        const bool t_vec = (rows % 16 == 0) && ((uintptr_t)out_t % 16 == 0);
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const int id = p * CAST_THREADS + t;
+            const int c = id >> 3, q = id & 7;  // tile column c (a row of out_t), 16-byte piece q
+            const int qsw = q ^ ((c >> 3) & 7);
+            const uint4 v = *(const uint4*)&tileT[c * (CAST_TILE / 4) + 4 * qsw];
+            const int64_t gc = c0 + c;
+            const int64_t gr = r0 + 16 * q;
+            if (gc < cols && gr < rows) {
+                uint8_t* dst = out_t + gc * rows + gr;
+                if (t_vec) {  // rows % 16 == 0 implies gr + 16 <= rows
+                    *(uint4*)dst = v;
+                } else {
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int i = 0; i < 16; i++)
+                        if (gr + i < rows) dst[i] = (uint8_t)((w[i >> 2] >> (8 * (i & 3))) & 0xffu);
+                }
+            }
+        }
+    }
+
+    if (amax_out) {
+        m = wave_max_u32(m);
+        const int wave = t >> 6, lane = t & 63;
+        if (lane == 0) red[wave] = m;
+        __syncthreads();
+        if (wave == 0) {
+            uint32_t v = lane < CAST_THREADS / 64 ? red[lane] : 0u;
+            m = wave_max_u32(v);
+        }
+        publish_amax_cast(m, ws, amax_out, DT);
+    }
+}
+
+__global__ void cast_zero_amax_kernel(float* amax_out) {
+    if (threadIdx.x == 0) *amax_out = 0.0f;
+}
+
+template <int DT, int PROD, int FMT>
+static int launch_cast2(bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
+                        const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, uint32_t* ws) {
+    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+    return check_hip(hipGetLastError(), "cast kernel launch");
+}
+
+template <int DT, int PROD>
+static int launch_cast1(int fmt, bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols,
+                        int64_t ld, const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev,
+                        uint32_t* ws) {
+    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+}
+
+}  // namespace f8mi
+
+using namespace f8mi;
+
+extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
+                         int product_dtype, int fp8_fmt, uint8_t* out, uint8_t* out_t, float* amax_dev,
+                         void* workspace, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (rows < 0 || cols < 0 || ld < cols) { set_error("f8mi_cast: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
+    if (in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
+    if (product_dtype != in_dtype && product_dtype != F8MI_FP32) { set_error("f8mi_cast: product_dtype must be the input dtype or fp32"); return F8MI_ERR_INVALID_ARG; }
+    if (!scale_dev) { set_error("f8mi_cast: null scale"); return F8MI_ERR_INVALID_ARG; }
+    if (!out && !out_t && !amax_dev) { set_error("f8mi_cast: no output requested"); return F8MI_ERR_INVALID_ARG; }
+    if (amax_dev && !workspace) { set_error("f8mi_cast: fused amax needs a workspace"); return F8MI_ERR_INVALID_ARG; }
+    if (rows == 0 || cols == 0) {
+        if (amax_dev) {
+            hipLaunchKernelGGL(cast_zero_amax_kernel, dim3(1), dim3(64), 0, stream, amax_dev);
+            return check_hip(hipGetLastError(), "cast_zero_amax_kernel");
+        }
+        return F8MI_OK;
+    }
+    if (!x) { set_error("f8mi_cast: null tensor"); return F8MI_ERR_INVALID_ARG; }
+    const int64_t ty = (rows + CAST_TILE - 1) / CAST_TILE, tx = (cols + CAST_TILE - 1) / CAST_TILE;
+    if (ty > 65535) { set_error("f8mi_cast: more than 65535*128 rows"); return F8MI_ERR_UNSUPPORTED; }
+    dim3 g((unsigned)tx, (unsigned)ty);
+    const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
+    const bool vec = ((uintptr_t)x % 16 == 0) && ((ld * esz) % 16 == 0);
+    const double n = (double)rows * (double)cols;
+    ProfScope prof(F8MI_K_CAST, n * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
+    uint32_t* ws = (uint32_t*)workspace;
+    if (in_dtype == F8MI_BF16) {
+        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+    }
+    if (in_dtype == F8MI_FP16) {
+        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+    }
+    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+}

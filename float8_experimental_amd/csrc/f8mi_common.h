@@ -1,0 +1,116 @@
+// Shared host/device helpers of libf8mi (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/f8mi.h"
+
+namespace f8mi {
+
+// ----------------------------------------------------------------- host side
+
+void set_error(const char* fmt, ...);
+int check_hip(hipError_t e, const char* what);
+
+// Profiling brackets (no-ops unless f8mi_prof_enable(1) was called).
+struct ProfScope {
+    int kernel;
+    double work;
+    hipStream_t stream;
+    void* rec;
+    ProfScope(int kernel, double work, hipStream_t stream);
+    ~ProfScope();
+};
+
+// workspace layout (uint32 words); every kernel leaves all words zero
+constexpr int WS_AMAX_BITS = 0;  // running max of |x| bit patterns
+constexpr int WS_TICKET = 1;     // blocks that have finished
+constexpr int WS_WORDS = 8;
+
+// ---------------------------------------------------------------- device side
+
+__device__ __forceinline__ float bits_to_float(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t float_to_bits(float f) { return __float_as_uint(f); }
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16 bits, round to nearest even; NaN -> quiet NaN.
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (f != f) ? 0x7fc0u : r;
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_float(float_to_bf16_bits(f)); }
+
+__device__ __forceinline__ float fp16_bits_to_float(uint32_t h) {
+    return __half2float(__ushort_as_half((unsigned short)h));
+}
+
+__device__ __forceinline__ float round_to_fp16(float f) { return __half2float(__float2half_rn(f)); }
+
+template <int DT>
+__device__ __forceinline__ float round_to(float f) {
+    if constexpr (DT == F8MI_BF16) return round_to_bf16(f);
+    else if constexpr (DT == F8MI_FP16) return round_to_fp16(f);
+    else return f;
+}
+
+__device__ __forceinline__ float round_to_rt(float f, int dt) {
+    if (dt == F8MI_BF16) return round_to_bf16(f);
+    if (dt == F8MI_FP16) return round_to_fp16(f);
+    return f;
+}
+
+__device__ __forceinline__ float fp8_max(int fmt) { return fmt == F8MI_E4M3FN ? 448.0f : 57344.0f; }
+
+// |x| bit pattern (as it sits in the dtype) -> the value widened to fp32.
+__device__ __forceinline__ float abs_bits_to_float(uint32_t bits, int dt) {
+    if (dt == F8MI_BF16) return bf16_bits_to_float(bits);
+    if (dt == F8MI_FP16) return fp16_bits_to_float(bits);
+    return __uint_as_float(bits);
+}
+
+// amax -> scale: clamp(amax, min=1e-12).reciprocal() * fmax, each step rounded to
+// `math_dt`, 1e-12 itself rounded to it first; optional clamp to fp16's max.
+__device__ __forceinline__ float amax_to_scale_dev(float amax, int math_dt, int fmt, int orig_is_fp16) {
+    float eps = round_to_rt(1e-12f, math_dt);
+    float c = (amax != amax) ? amax : (amax < eps ? eps : amax);
+    float r = round_to_rt(__fdiv_rn(1.0f, c), math_dt);
+    float s = round_to_rt(__fmul_rn(r, fp8_max(fmt)), math_dt);
+    if (orig_is_fp16 && s > 65504.0f) s = 65504.0f;
+    return s;
+}
+
+// Two fp32 -> two OCP fp8 bytes (low 16 bits of the result), round to nearest
+// even via the gfx950 conversion instructions.  Inputs must already be clamped
+// to the finite range or be NaN; NaN gives a NaN code.
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt2_fp8(float a, float b) {
+    uint32_t r;
+    if constexpr (FMT == F8MI_E4M3FN) r = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    else r = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    return r & 0xffffu;
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 16-byte streaming load (data is used once: keep it out of the way of reused lines)
+__device__ __forceinline__ uint4 load_nt16(const void* p) {
+    u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// wave-wide max of a uint32 (wave64)
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        uint32_t o = (uint32_t)__shfl_xor((int)v, off, 64);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+}  // namespace f8mi

@@ -1,0 +1,165 @@
+/*
+ * f8mi.h -- C ABI of libf8mi.so: the Float8Linear training hot path of
+ * pytorch-labs/float8_experimental as hand-written gfx950 (MI355X) kernels.
+ *
+ * Conventions
+ *   - Every pointer named `*_dev`, every tensor pointer and every workspace is
+ *     DEVICE memory owned by the caller.  The library never allocates, frees or
+ *     synchronises; every call only enqueues kernels on `stream` (a
+ *     hipStream_t passed as void*; NULL = the default stream).
+ *   - Calls are re-entrant and may come from any host thread (autograd runs the
+ *     backward on its own thread).
+ *   - Return value: F8MI_OK or a negative F8MI_ERR_* code; f8mi_last_error()
+ *     gives the calling thread's last message.
+ *   - "scale" always has the reference's meaning: high precision * scale = fp8
+ *     range (float8_tensor.py:252-255 of the reference).
+ *
+ * Paths cited below are relative to the reference checkout
+ * (pytorch-labs/float8_experimental).
+ */
+#ifndef F8MI_H
+#define F8MI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define F8MI_VERSION 100
+
+#define F8MI_OK 0
+#define F8MI_ERR_INVALID_ARG (-1) /* null pointer, negative size, unknown enum            */
+#define F8MI_ERR_UNSUPPORTED (-2) /* valid request this build does not implement          */
+#define F8MI_ERR_HIP (-3)         /* a HIP runtime call failed (launch, event, ...)       */
+#define F8MI_ERR_ARCH (-4)        /* the current device is not gfx950                     */
+
+/* element type of a high-precision tensor, and the dtype arithmetic is rounded to */
+#define F8MI_BF16 0
+#define F8MI_FP16 1
+#define F8MI_FP32 2
+
+/* OCP fp8 formats (torch.float8_e4m3fn / torch.float8_e5m2; float8_utils.py:31-32) */
+#define F8MI_E4M3FN 0
+#define F8MI_E5M2 1
+
+/* kernel ids for the profiling counters */
+#define F8MI_K_AMAX 0
+#define F8MI_K_CAST 1
+#define F8MI_K_GEMM 2
+#define F8MI_K_SYNC 3
+#define F8MI_K_COUNT 4
+
+int f8mi_version(void);
+const char* f8mi_last_error(void);
+
+/* Fills CU count, LDS bytes per workgroup and the gcn arch name of HIP device `device`.
+ * Returns F8MI_ERR_ARCH when it is not a gfx950. */
+int f8mi_device_info(int device, int* cu_count, int* lds_bytes, char* arch, int arch_len);
+
+/* Bytes of the small device workspace the reducing kernels need.  The caller
+ * zero-fills it ONCE; every kernel leaves it zeroed again.  One workspace must
+ * not be shared by calls that can overlap in time (use one per stream). */
+size_t f8mi_workspace_bytes(void);
+
+/*
+ * amax = max|x| and the fp8 scale derived from it, in one pass over x.
+ * Replaces tensor_to_amax (float8_utils.py:102-112) + amax_to_scale
+ * (float8_utils.py:35-57), i.e. tensor_to_scale (float8_utils.py:115-120).
+ *   x          rows x cols elements of `in_dtype`, row stride `ld` elements
+ *   math_dtype dtype each step of `fmax / clamp(amax, 1e-12)` is rounded to:
+ *              `in_dtype` for dynamic scaling (the reference computes the scale
+ *              in the tensor's dtype), F8MI_FP32 for delayed-scaling buffers
+ *   orig_is_fp16  clamp the scale to 65504 (float8_utils.py:54-55)
+ *   amax_dev   out, 1 float (the amax widened to fp32), may be NULL
+ *   scale_dev  out, 1 float, may be NULL
+ * NaN anywhere in x gives NaN amax and NaN scale, like torch.max.
+ */
+int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt,
+                    int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
+                    void* stream);
+
+/*
+ * Saturated cast to fp8: bytes = fp8(clamp(x * scale, -fmax, fmax)), round to
+ * nearest even.  Replaces _ToFloat8ConstrFunc.forward (float8_tensor.py:139-191)
+ * + to_fp8_saturated (float8_utils.py:123-139), and the fp8 transpose copies
+ * that preprocess_addmm makes for the backward GEMMs (float8_ops.py:131-155).
+ *   scale_dev      1 float in device memory
+ *   product_dtype  dtype `x * scale` is rounded to before clamp + conversion:
+ *                  `in_dtype` when the reference's scale is a 0-dim tensor
+ *                  (dynamic scaling), F8MI_FP32 when it is the [1]-shaped buffer
+ *                  of delayed scaling or x is fp32
+ *   out            rows x cols bytes, dense row-major; may be NULL
+ *   out_t          cols x rows bytes, dense (the transpose); may be NULL
+ *   amax_dev       if not NULL, max|x| of THIS call is stored there (fused
+ *                  amax for hp_tensor_to_float8_delayed,
+ *                  float8_scaling_utils.py:65-96); needs `workspace`
+ */
+int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
+              int product_dtype, int fp8_fmt, uint8_t* out, uint8_t* out_t, float* amax_dev, void* workspace,
+              void* stream);
+
+/*
+ * C[m][n] = (sum_k A[m][k] * Bt[n][k]) * (1/scale_a) * (1/scale_b) (+ bias[n]),
+ * fp32 accumulation on the fp8 matrix cores.  Replaces addmm_float8_unwrapped
+ * -> torch._scaled_mm (float8_python_api.py:24-64) as reached from float8_mm
+ * (float8_ops.py:158-190).  Both operands are contiguous along k (A row-major,
+ * B column-major in the reference's words): forward x*W^T, grad_input dY*W and
+ * grad_weight dY^T*x all have this form once the transposed copies exist.
+ * Any m, n, k >= 0 is accepted (ragged edges are handled in the kernel).
+ *   a_fmt/b_fmt   F8MI_E4M3FN / F8MI_E5M2 per operand
+ *   lda/ldb       row strides in bytes (>= k)
+ *   scale_a_dev, scale_b_dev   the operands' forward scales (1 float each)
+ *   c_dtype       F8MI_BF16 / F8MI_FP16 / F8MI_FP32, ldc in elements
+ *   bias_dev      n elements of c_dtype, or NULL
+ */
+int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fmt, int64_t ldb, int64_t m,
+                 int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
+                 int64_t ldc, const void* bias_dev, void* stream);
+
+/* One (layer, tensor) row of the delayed-scaling bookkeeping; all device pointers. */
+typedef struct f8mi_sync_entry {
+    float* amax;    /* [1]        fp8_amax_*          */
+    float* history; /* [hist_len] fp8_amax_history_*  */
+    float* scale;   /* [1]        fp8_scale_*         */
+    int64_t fp8_fmt;
+} f8mi_sync_entry;
+
+/*
+ * For each of the n entries: S = roll(history, 1); S[0] = amax;
+ * scale = fmax * (1 / clamp(max(S), 1e-12)) in fp32 (<= 65504 if orig_is_fp16).
+ * Replaces the body of sync_float8_amax_and_scale_history
+ * (float8_linear_utils.py:287-319: _update_history_stack :37-56 and
+ * amax_history_to_scale_stack, float8_utils.py:80-99) in one launch.
+ * writeback_history = 0 reproduces the reference, which rolls a stacked copy
+ * and leaves each layer's history buffer untouched; 1 stores S back.
+ * `entries_dev` is a device array of n f8mi_sync_entry.
+ */
+int f8mi_sync(const f8mi_sync_entry* entries_dev, int n, int hist_len, int orig_is_fp16, int writeback_history,
+              void* stream);
+
+/*
+ * First-iteration initialisation of one tensor's buffers
+ * (_maybe_initialize_amaxes_scales_for_float8_cast, float8_scaling_utils.py:99-125):
+ * history[0] = *amax; *scale = fmax * (1 / clamp(max(history), 1e-12)).
+ * `amax_dev` must already hold this step's amax (f8mi_amax_scale).
+ */
+int f8mi_delayed_init(const float* amax_dev, float* history_dev, float* scale_dev, int hist_len, int fp8_fmt,
+                      int orig_is_fp16, void* stream);
+
+/*
+ * Optional per-kernel timing with HIP events on the launch stream.  While
+ * enabled every launch of kernel class `kernel` (F8MI_K_*) is bracketed by two
+ * events; f8mi_prof_read synchronises them and returns launches, summed
+ * milliseconds and summed algorithmic work (bytes for amax/cast/sync, flop for
+ * gemm).  Off by default; meant for benchmarks, not for training loops.
+ */
+int f8mi_prof_enable(int on);
+int f8mi_prof_reset(void);
+int f8mi_prof_read(int kernel, uint64_t* launches, double* total_ms, double* total_work);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* F8MI_H */

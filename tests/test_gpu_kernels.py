@@ -1,0 +1,393 @@
+"""Parity of the HIP kernels (through the C ABI) with the CPU oracle.  Needs an MI355X.
+
+Bars: amax, scales and fp8 bytes bit-exact (NaN codes may differ in the sign
+bit); GEMM within a stated tolerance of the emulated fp32 product.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import CODE_DT, F8, TORCH_DT, fp8_bytes, np_for_c, same_bytes_mod_nan_sign
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def nat():
+    if not torch.cuda.is_available():
+        pytest.fail("these tests need a GPU (run with -m gpu on an MI355X box)")
+    from float8_experimental_amd import _native
+
+    _native.lib()
+    return _native
+
+
+def _oracles():
+    from oracle import c_oracle as co
+    from oracle import torch_oracle as to
+
+    return co, to
+
+
+def heavy(shape, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    t = torch.distributions.StudentT(3.0).sample(shape)
+    mask = torch.rand(shape, generator=g) < 0.001
+    return torch.where(mask, t * 1000, t).to(dtype)
+
+
+# ------------------------------------------------------------------ K1 amax
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(1,), (7,), (4, 8), (33, 47), (257, 1031), (1024, 4096), (3, 5, 64)])
+def test_amax_scale_matches_oracle(nat, dt, shape):
+    co, to = _oracles()
+    torch.manual_seed(hash((dt, shape)) % 1000)
+    x = heavy(shape, TORCH_DT[dt], 1)
+    xd = x.to(DEV)
+    for fmt, (code, tdt) in F8.items():
+        amax, scale = nat.amax_scale(xd, tdt)
+        want_a = to.tensor_to_amax(x).float()
+        want_s = to.tensor_to_scale(x, tdt)
+        assert amax.cpu().view(torch.int32).item() == want_a.view(torch.int32).item()
+        assert scale.cpu().view(torch.int32).item() == want_s.view(torch.int32).item(), (dt, fmt, shape)
+        # fp32 math (delayed-scaling buffers)
+        _, s32 = nat.amax_scale(xd, tdt, math_dtype=torch.float32)
+        want = to.amax_to_scale(want_a, tdt, TORCH_DT[dt])
+        assert s32.cpu().view(torch.int32).item() == want.view(torch.int32).item()
+
+
+def test_amax_strided_rows_and_unaligned_views(nat):
+    co, to = _oracles()
+    torch.manual_seed(3)
+    base = torch.randn(64, 300).to(torch.bfloat16)
+    based = base.to(DEV)
+    for view in (lambda t: t[:, 3:259], lambda t: t[5:40, 1:2], lambda t: t[:, ::2], lambda t: t.t()):
+        x, xd = view(base), view(based)
+        amax, scale = nat.amax_scale(xd, torch.float8_e4m3fn)
+        assert amax.item() == to.tensor_to_amax(x).float().item()
+        assert scale.item() == to.tensor_to_scale(x, torch.float8_e4m3fn).item()
+
+
+def test_amax_specials(nat):
+    co, to = _oracles()
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        z = torch.zeros(1000, dtype=dt, device=DEV)
+        for f8 in (torch.float8_e4m3fn, torch.float8_e5m2):
+            a, s = nat.amax_scale(z, f8)
+            assert a.item() == 0.0
+            assert s.item() == to.tensor_to_scale(torch.zeros(4, dtype=dt), f8).item()
+        z[77] = float("nan")
+        a, s = nat.amax_scale(z, torch.float8_e4m3fn)
+        assert torch.isnan(a).item() and torch.isnan(s).item()
+        z[77] = float("-inf")
+        a, s = nat.amax_scale(z, torch.float8_e4m3fn)
+        assert a.item() == float("inf") and s.item() == 0.0
+    # the workspace is left clean: a later call on other data is unaffected
+    a, _ = nat.amax_scale(torch.full((10,), 0.5, dtype=torch.bfloat16, device=DEV), torch.float8_e4m3fn)
+    assert a.item() == 0.5
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+def test_scale_math_sweep_16bit(nat, dt):
+    """Scale arithmetic in the tensor's own dtype over a sweep of amax bit patterns."""
+    co, to = _oracles()
+    top = 0x7C00 if dt == "fp16" else 0x7F80
+    pats = np.unique(np.concatenate([np.arange(0, top, 37), np.array([0, 1, 2, top - 1, 0x3F80, 0x3C00])])).astype(np.uint16)
+    for fmt, (code, tdt) in F8.items():
+        for p in pats[:: 1 if dt == "bf16" else 2]:
+            x = torch.from_numpy(np.array([0, p, 0], np.uint16).view(np.int16)).view(TORCH_DT[dt]).to(DEV)
+            a, s = nat.amax_scale(x, tdt)
+            want = co.amax_to_scale(a.item(), CODE_DT[dt], code, dt == "fp16")
+            assert np.float32(s.item()).view(np.uint32) == np.float32(want).view(np.uint32), (dt, fmt, hex(int(p)))
+
+
+# ------------------------------------------------------------------ K2 cast
+
+
+def _ref_cast(x_cpu, scale_cpu, tdt, delayed):
+    _, to = _oracles()
+    s = scale_cpu.reshape(1) if delayed else scale_cpu.reshape(())
+    return fp8_bytes(to.cast_to_fp8(x_cpu, s, tdt))
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_cast_every_16bit_pattern(nat, dt, fmt):
+    code, tdt = F8[fmt]
+    allb = np.arange(65536, dtype=np.uint16)
+    x = torch.from_numpy(allb.view(np.int16).copy()).view(TORCH_DT[dt]).reshape(256, 256)
+    xd = x.to(DEV)
+    scales = [1.0, 448.0 / 3.0, 0.0123, 57344.0 / 0.011, 1e-6, 3.3e4, 2.0**-20, 1.7]
+    for s in scales:
+        for delayed in (False, True):
+            sc = torch.tensor(s, dtype=torch.float32)
+            if dt == "fp16" and not delayed and s > 65504:
+                continue
+            want = _ref_cast(x, sc, tdt, delayed)
+            out, out_t = nat.cast(xd, sc.to(DEV), tdt, product_dtype=torch.float32 if delayed else TORCH_DT[dt],
+                                  want_out_t=True)
+            got = fp8_bytes(out)
+            assert same_bytes_mod_nan_sign(got, want), (dt, fmt, s, delayed, int((got != want).sum()))
+            assert np.array_equal(fp8_bytes(out_t), got.T)
+
+
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_cast_fp32_bit_patterns(nat, fmt):
+    code, tdt = F8[fmt]
+    rng = np.random.default_rng(5)
+    bits = np.concatenate([np.arange(0, 2**32, 8191, dtype=np.uint64).astype(np.uint32)[: 512 * 1024],
+                           rng.integers(0, 2**32, size=512 * 1024, dtype=np.uint64).astype(np.uint32)])
+    x = torch.from_numpy(bits.view(np.float32).copy()).reshape(1024, 1024)
+    xd = x.to(DEV)
+    for s in (1.0, 0.37, 1234.5):
+        sc = torch.tensor(s, dtype=torch.float32)
+        want = _ref_cast(x, sc, tdt, True)
+        out, out_t = nat.cast(xd, sc.to(DEV), tdt, want_out_t=True)
+        assert same_bytes_mod_nan_sign(fp8_bytes(out), want)
+        assert np.array_equal(fp8_bytes(out_t), fp8_bytes(out).T)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 129), (129, 1), (16, 16), (33, 47), (128, 128), (257, 131), (130, 1000),
+                                   (1000, 136), (4099, 1000), (2, 3, 40)])
+def test_cast_shapes_dynamic_and_delayed(nat, dt, shape):
+    co, to = _oracles()
+    x = heavy(shape, TORCH_DT[dt], 2)
+    xd = x.to(DEV)
+    x2 = x.reshape(-1, shape[-1])
+    for fmt, (code, tdt) in F8.items():
+        s = to.tensor_to_scale(x, tdt)
+        # dynamic: product in the tensor's dtype
+        out, out_t = nat.cast(xd, s.to(DEV), tdt, want_out_t=True)
+        want = fp8_bytes(to.cast_to_fp8(x, s, tdt))
+        assert out.shape == x.shape and out_t.shape == (x2.shape[1], x2.shape[0])
+        assert np.array_equal(fp8_bytes(out), want), (dt, fmt, shape)
+        assert np.array_equal(fp8_bytes(out_t), want.reshape(x2.shape).T)
+        # delayed: [1]-shaped scale that saturates part of the tensor, amax fused
+        s1 = (s * 2.5).reshape(1)
+        amax = torch.full((1,), -1.0, dtype=torch.float32, device=DEV)
+        out, out_t = nat.cast(xd, s1.to(DEV), tdt, product_dtype=torch.float32, want_out_t=True, amax_out=amax)
+        want = fp8_bytes(to.cast_to_fp8(x, s1, tdt))
+        assert np.array_equal(fp8_bytes(out), want), (dt, fmt, shape, "delayed")
+        assert np.array_equal(fp8_bytes(out_t), want.reshape(x2.shape).T)
+        assert amax.item() == to.tensor_to_amax(x).float().item()
+        # only the transposed copy
+        _, only_t = nat.cast(xd, s1.to(DEV), tdt, product_dtype=torch.float32, want_out=False, want_out_t=True)
+        assert np.array_equal(fp8_bytes(only_t), want.reshape(x2.shape).T)
+
+
+def test_cast_row_strided_and_c_oracle(nat):
+    co, to = _oracles()
+    base = heavy((70, 400), torch.bfloat16, 4)
+    x, xd = base[:, 8:264], base.to(DEV)[:, 8:264]     # 16-byte aligned rows, ld != cols
+    y, yd = base[3:, 5:206], base.to(DEV)[3:, 5:206]   # unaligned
+    for t, td in ((x, xd), (y, yd)):
+        s = to.tensor_to_scale(t, torch.float8_e4m3fn)
+        out, out_t = nat.cast(td, s.to(DEV), torch.float8_e4m3fn, want_out_t=True)
+        want_c, want_ct = co.cast(np_for_c(t), co.BF16, s.item(), co.BF16, co.E4M3FN, transpose=True)
+        assert np.array_equal(fp8_bytes(out), want_c) and np.array_equal(fp8_bytes(out_t), want_ct)
+
+
+def test_cfg1_dy_ones(nat):
+    """BASELINE config 1: dY = ones -> scale 57344, every e5m2 byte 0x7B."""
+    dy = torch.ones(2048, 4096, dtype=torch.bfloat16, device=DEV)
+    a, s = nat.amax_scale(dy, torch.float8_e5m2)
+    assert a.item() == 1.0 and s.item() == 57344.0
+    out, out_t = nat.cast(dy, s, torch.float8_e5m2, want_out_t=True)
+    assert bool((out.view(torch.uint8) == 0x7B).all()) and bool((out_t.view(torch.uint8) == 0x7B).all())
+
+
+def test_golden_cast_fixtures_on_gpu(nat):
+    from tests.helpers import from_bits, load
+
+    g = load("casts")
+    for case in sorted({k[:-2] for k in g.files if k.endswith(".x")}):
+        dt = case.split(".")[0]
+        x = from_bits(g[case + ".x"], dt).to(DEV)
+        for fmt, (code, tdt) in F8.items():
+            a, s = nat.amax_scale(x, tdt)
+            assert np.float32(s.item()).view(np.uint32) == g[f"{case}.{fmt}.scale"].view(np.uint32), (case, fmt)
+            out, _ = nat.cast(x, s, tdt)
+            assert np.array_equal(fp8_bytes(out), g[f"{case}.{fmt}.dyn"]), (case, fmt)
+            s1 = torch.from_numpy(g[f"{case}.{fmt}.scale1"].copy()).to(DEV)
+            out, _ = nat.cast(x, s1, tdt, product_dtype=torch.float32)
+            assert np.array_equal(fp8_bytes(out), g[f"{case}.{fmt}.del"]), (case, fmt)
+
+
+# ------------------------------------------------------------------ K3 gemm
+
+
+def _rand_fp8(shape, tdt, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    v = torch.randn(shape, generator=g) * scale
+    fmax = torch.finfo(tdt).max
+    return v.clamp(-fmax, fmax).to(tdt)
+
+
+def _gemm_check(nat, m, n, k, a_fmt, b_fmt, out_dt, seed=0, bias=False, sa=3.0, sb=0.5):
+    co, to = _oracles()
+    ta, tb = F8[a_fmt][1], F8[b_fmt][1]
+    a = _rand_fp8((m, k), ta, seed, 4.0)
+    bt = _rand_fp8((n, k), tb, seed + 1, 4.0)
+    sa_t, sb_t = torch.tensor(sa), torch.tensor(sb)
+    bias_t = (torch.randn(n) * 3).to(out_dt) if bias else None
+    got = nat.gemm_nt(a.to(DEV), sa_t.to(DEV), bt.to(DEV), sb_t.to(DEV), out_dt,
+                      bias=bias_t.to(DEV) if bias else None).cpu().double()
+    ad, bd = a.double() / sa, bt.double() / sb
+    exact = ad @ bd.T
+    if bias:
+        exact = exact + bias_t.double()
+    bound = ad.abs() @ bd.abs().T + (bias_t.double().abs() if bias else 0)  # elementwise magnitude of the sum
+    eps_out = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-23}[out_dt]
+    # stated tolerance: one output rounding + fp32 accumulation noise relative to the magnitude of the terms
+    tol = eps_out * exact.abs() + 2e-5 * bound + 1e-30
+    err = (got - exact).abs()
+    worst = (err / tol).max().item()
+    assert worst <= 1.0, (m, n, k, a_fmt, b_fmt, out_dt, worst)
+    # and against the reference's emulated op itself (fp32 mm on CPU), north-star bar 1e-2
+    emu = to.mm_emulated(a, sa_t, bt.t(), sb_t, out_dt)
+    if bias:
+        emu = emu + bias_t
+    rel = ((got - emu.double()).abs() / (emu.double().abs() + 1e-2 * bound.max())).max().item()
+    assert rel <= 1e-2, (m, n, k, rel)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (256, 256, 256), (512, 768, 384), (16, 32, 16), (1, 1, 1),
+                                   (300, 520, 200), (257, 255, 129), (64, 4096, 1024), (1000, 3000, 4099 // 4 * 4),
+                                   (129, 77, 4097), (40, 50, 1000), (2048, 512, 2048)])
+def test_gemm_shapes(nat, m, n, k):
+    _gemm_check(nat, m, n, k, "e4m3", "e4m3", torch.bfloat16, seed=m + n + k)
+
+
+@pytest.mark.parametrize("a_fmt,b_fmt", [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2"), ("e5m2", "e5m2")])
+@pytest.mark.parametrize("out_dt", [torch.bfloat16, torch.float16, torch.float32])
+def test_gemm_formats_and_output_dtypes(nat, a_fmt, b_fmt, out_dt):
+    _gemm_check(nat, 384, 320, 448, a_fmt, b_fmt, out_dt, seed=7, bias=(out_dt != torch.float16))
+
+
+def test_gemm_closed_forms(nat):
+    one4 = torch.tensor([1.0]).to(torch.float8_e4m3fn)
+    # identity: A @ I = A exactly (every fp8 value is a bf16 value)
+    a = _rand_fp8((300, 256), torch.float8_e4m3fn, 3, 50.0)
+    eye = torch.eye(256).to(torch.float8_e4m3fn)
+    s1 = torch.ones((), device=DEV)
+    out = nat.gemm_nt(a.to(DEV), s1, eye.to(DEV), s1, torch.bfloat16)
+    assert torch.equal(out.cpu().float(), a.float())
+    # all ones: k / (sa * sb)
+    a = torch.ones(70, 1000).to(torch.float8_e5m2)
+    b = torch.ones(90, 1000).to(torch.float8_e4m3fn)
+    out = nat.gemm_nt(a.to(DEV), torch.tensor(2.0, device=DEV), b.to(DEV), torch.tensor(4.0, device=DEV), torch.float32)
+    assert bool((out == 125.0).all())
+    # one-hot rows pick single columns (catches a transposed or permuted operand)
+    a = torch.zeros(64, 512)
+    idx = torch.arange(64) * 7 % 512
+    a[torch.arange(64), idx] = 2.0
+    bt = _rand_fp8((96, 512), torch.float8_e4m3fn, 9, 8.0)
+    out = nat.gemm_nt(a.to(torch.float8_e4m3fn).to(DEV), s1, bt.to(DEV), s1, torch.float32).cpu()
+    assert torch.equal(out, 2.0 * bt.float()[:, idx].t())
+    # zero-padding the reduction changes nothing (reference test_base.py:477-552 pads to 16)
+    a = _rand_fp8((50, 41), torch.float8_e4m3fn, 11)
+    bt = _rand_fp8((128, 41), torch.float8_e4m3fn, 12)
+    o1 = nat.gemm_nt(a.to(DEV), s1, bt.to(DEV), s1, torch.float32)
+    ap = torch.nn.functional.pad(a.view(torch.uint8), (0, 7)).view(torch.float8_e4m3fn)
+    bp = torch.nn.functional.pad(bt.view(torch.uint8), (0, 7)).view(torch.float8_e4m3fn)
+    o2 = nat.gemm_nt(ap.to(DEV), s1, bp.to(DEV), s1, torch.float32)
+    assert torch.equal(o1, o2)
+    # k = 0: the empty sum
+    o = nat.gemm_nt(torch.empty(5, 0, dtype=torch.float8_e4m3fn, device=DEV), s1,
+                    torch.empty(6, 0, dtype=torch.float8_e4m3fn, device=DEV), s1, torch.bfloat16)
+    assert o.shape == (5, 6) and bool((o == 0).all())
+
+
+def test_gemm_strided_operands(nat):
+    co, to = _oracles()
+    a = _rand_fp8((200, 512), torch.float8_e4m3fn, 21)
+    bt = _rand_fp8((300, 512), torch.float8_e4m3fn, 22)
+    ad, bd = a.to(DEV), bt.to(DEV)
+    s1 = torch.ones((), device=DEV)
+    # row-strided views (ld > k), aligned and not
+    for sl in (slice(0, 256), slice(16, 400), slice(3, 260)):
+        out = nat.gemm_nt(ad[:, sl], s1, bd[:, sl], s1, torch.float32).cpu()
+        want = a[:, sl].float() @ bt[:, sl].float().t()
+        torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-3)
+
+
+# ------------------------------------------------------------------ K4 sync
+
+
+def test_sync_and_init_match_oracle(nat):
+    co, to = _oracles()
+    rng = np.random.default_rng(0)
+    n, H = 999, 16
+    amax = (np.abs(rng.standard_normal(n)) * 10.0 ** rng.integers(-14, 5, n)).astype(np.float32)
+    hist = (np.abs(rng.standard_normal((n, H))) * 10.0 ** rng.integers(-14, 5, (n, 1))).astype(np.float32)
+    hist[::7] = 0
+    amax[:3] = [0.0, 448.0, np.nan]
+    fmts = rng.integers(0, 2, n)
+    for fp16 in (False, True):
+        for wb in (False, True):
+            a_d = torch.from_numpy(amax.copy()).to(DEV).reshape(n, 1)
+            h_d = torch.from_numpy(hist.copy()).to(DEV)
+            s_d = torch.zeros(n, 1, device=DEV)
+            table = nat.sync_table(((a_d[i], h_d[i], s_d[i], (torch.float8_e4m3fn, torch.float8_e5m2)[fmts[i]])
+                                    for i in range(n)), torch.device(DEV))
+            nat.sync(table, H, fp16, wb)
+            got_s, got_h = s_d.cpu().numpy().reshape(-1), h_d.cpu().numpy()
+            for i in range(n):
+                h = hist[i].copy()
+                want = co.sync_entry(amax[i], h, int(fmts[i]), fp16, wb)
+                assert np.float32(got_s[i]).view(np.uint32) == np.float32(want).view(np.uint32) or (np.isnan(want) and np.isnan(got_s[i])), i
+                assert np.array_equal(got_h[i], h, equal_nan=True), (i, wb)
+    # init
+    for i in range(0, 60):
+        h = hist[i].copy()
+        a_d = torch.tensor([amax[i]], device=DEV)
+        h_d = torch.from_numpy(h.copy()).to(DEV)
+        s_d = torch.zeros(1, device=DEV)
+        nat.delayed_init(a_d, h_d, s_d, (torch.float8_e4m3fn, torch.float8_e5m2)[fmts[i]], False)
+        want = co.delayed_init(amax[i], h, int(fmts[i]), False)
+        assert np.array_equal(h_d.cpu().numpy(), h, equal_nan=True)
+        assert np.float32(s_d.item()).view(np.uint32) == np.float32(want).view(np.uint32) or np.isnan(want)
+
+
+# ------------------------------------------- full-size properties (config 2)
+
+
+def test_full_size_properties_llama70b_wo(nat):
+    """M=16384, K=N=8192: size-independent properties where the oracle is too slow."""
+    torch.manual_seed(0)
+    M, K, N = 16384, 8192, 8192
+    x = torch.randn(M, K, device=DEV, dtype=torch.bfloat16)
+    w = (torch.rand(N, K, device=DEV, dtype=torch.float32) * 2 - 1).mul_(K**-0.5).to(torch.bfloat16)
+    ax, sx = nat.amax_scale(x, torch.float8_e4m3fn)
+    aw, sw = nat.amax_scale(w, torch.float8_e4m3fn)
+    assert ax.item() == x.abs().max().float().item() and aw.item() == w.abs().max().float().item()
+    x8, x8t = nat.cast(x, sx, torch.float8_e4m3fn, want_out_t=True)
+    w8, w8t = nat.cast(w, sw, torch.float8_e4m3fn, want_out_t=True)
+    assert torch.equal(x8t.view(torch.uint8), x8.view(torch.uint8).t().contiguous())
+    assert torch.equal(w8t.view(torch.uint8), w8.view(torch.uint8).t().contiguous())
+    # the cast is the same function of (x, scale) everywhere: torch's own ops on the GPU agree byte for byte
+    ref = (x * sx).clamp(-448, 448).to(torch.float8_e4m3fn)
+    assert torch.equal(ref.view(torch.uint8), x8.view(torch.uint8))
+    # idempotence: re-casting the dequantised tensor at scale 1 gives the same bytes
+    one = torch.ones((), device=DEV)
+    again, _ = nat.cast(x8.to(torch.bfloat16), one, torch.float8_e4m3fn)
+    assert torch.equal(again.view(torch.uint8), x8.view(torch.uint8))
+    # GEMM: checksum of checksums in fp64, and exact linearity in power-of-two scales
+    y = nat.gemm_nt(x8, sx, w8, sw, torch.float32)
+    col = (x8.double().sum(0) / sx.double()) @ (w8.double().t() / sw.double())
+    torch.testing.assert_close(y.double().sum(0), col, rtol=1e-4, atol=1e-4 * col.abs().max().item())
+    row = (x8.double() / sx.double()) @ (w8.double().sum(0) / sw.double())
+    torch.testing.assert_close(y.double().sum(1), row, rtol=1e-4, atol=1e-4 * row.abs().max().item())
+    y2 = nat.gemm_nt(x8, sx * 2, w8, sw * 4, torch.float32)
+    assert torch.equal(y2 * 8, y)
+    # a 64 x 64 corner against the emulated product computed in fp64
+    sub = (x8[:64].double() / sx.double()) @ (w8[:64].double().t() / sw.double())
+    torch.testing.assert_close(y[:64, :64].double(), sub, rtol=1e-4, atol=1e-4)
+    # grad_weight-shaped product from the transposed copies: (x^T x)[i][j], symmetric by construction
+    g = nat.gemm_nt(x8t[:512], sx, x8t[:768], sx, torch.float32)
+    torch.testing.assert_close(g[:, :512], g[:, :512].t(), rtol=1e-5, atol=1e-3)
