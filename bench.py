@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Float8Linear fwd+bwd throughput at LLaMa-2-70B linear shapes on one MI355X.
+
+One "step" = forward + backward (dynamic scaling on input, weight and grad_output)
+through each of the four 70B linear shapes at M = 16384 tokens, inputs resident in
+HBM.  Prints ONE JSON line: whole-job TFLOP/s (3 * 2*M*K*N flop per shape, the
+reference benchmark's convention), the fp8 GEMM kernel's roofline position measured
+with HIP events around every launch inside the timed region, the amax / cast
+kernels' HBM figures, bf16 nn.Linear on the same GPU, and the CPU oracle timed on
+a bounded sample on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+SHAPES = [  # (name, K, N) at M tokens
+    ("wqkv", 8192, 10240),
+    ("wo", 8192, 8192),
+    ("w13", 8192, 57344),
+    ("w2", 28672, 8192),
+]
+M_TOKENS = 16384
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=5)
+    p.add_argument("--warmup", type=int, default=2)
+    p.add_argument("--m", type=int, default=M_TOKENS, help="tokens per step (default: the benchmark's 16384)")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-bf16", action="store_true")
+    p.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the oracle sample")
+    return p.parse_args()
+
+
+def make_layers(torch, f8, m, device):
+    layers = []
+    for name, k, n in SHAPES:
+        lin = torch.nn.Linear(k, n, bias=False, device=device, dtype=torch.bfloat16)  # kaiming-uniform init
+        mod = f8.Float8Linear.from_float(lin, config=f8.Float8LinearConfig())
+        x = torch.randn(m, k, device=device, dtype=torch.bfloat16).requires_grad_()
+        dy = (torch.randn(m, n, device=device, dtype=torch.float32) * 1e-2).to(torch.bfloat16)
+        layers.append((name, k, n, lin, mod, x, dy))
+    return layers
+
+
+def step(layers, use_fp8=True):
+    for name, k, n, lin, mod, x, dy in layers:
+        x.grad = None
+        lin.weight.grad = None
+        y = (mod if use_fp8 else lin)(x)
+        y.backward(dy)
+
+
+def timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def cpu_baseline(torch, target_s):
+    """The oracle's emulate=True restatement (fp32 dequant + torch.mm on the host) on a slice of the wo shape."""
+    from oracle import torch_oracle as to
+
+    k = n = 8192
+    torch.manual_seed(0)
+    w = (torch.rand(n, k) * 2 - 1).mul_(k**-0.5).to(torch.bfloat16)
+
+    def run(m):
+        x = torch.randn(m, k).to(torch.bfloat16)
+        dy = (torch.randn(m, n) * 1e-2).to(torch.bfloat16)
+        t0 = time.perf_counter()
+        to.linear_fwd_bwd_dynamic(x, w, dy)
+        return time.perf_counter() - t0
+
+    run(256)  # warm the BLAS threads
+    t_small = run(512)
+    m = 512
+    while m < M_TOKENS and t_small * (2 * m / 512) <= target_s:
+        m *= 2
+    t = run(m)
+    flop = 3 * 2.0 * m * k * n
+    return {
+        "value": flop / t / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle.torch_oracle.linear_fwd_bwd_dynamic (amax+scale, saturated casts, 3 emulated fp32 GEMMs) on "
+                  f"M={m} of {M_TOKENS} tokens of the wo shape K=N=8192, one run, {t:.2f} s",
+        "seconds": t,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build drives ONE GPU (no collectives in the path); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import float8_experimental_amd as f8
+    from float8_experimental_amd import _native
+
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    _native.lib()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    m = args.m
+    layers = make_layers(torch, f8, m, dev)
+    flop_per_shape = {name: 3 * 2.0 * m * k * n for name, k, n, *_ in layers}
+    flop_step = sum(flop_per_shape.values())
+
+    # ---- the timed region: K steps, every kernel launch bracketed by HIP events on its stream
+    for _ in range(args.warmup):
+        step(layers)
+    torch.cuda.synchronize()
+    _native.prof_reset()
+    _native.prof_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(layers)
+    torch.cuda.synchronize()
+    sec_step = (time.perf_counter() - t0) / args.steps
+    _native.prof_enable(False)
+    prof = {name: _native.prof_read(kid) for name, kid in
+            (("amax", _native.K_AMAX), ("cast", _native.K_CAST), ("gemm", _native.K_GEMM))}
+    _native.prof_reset()
+
+    n_gemm, ms_gemm, flop_gemm = prof["gemm"]
+    gemm_tflops = flop_gemm / (ms_gemm * 1e-3) / 1e12 if ms_gemm > 0 else 0.0
+    hbm = {}
+    for kname in ("amax", "cast"):
+        cnt, ms, nbytes = prof[kname]
+        hbm[kname] = {"launches": cnt, "GB/s": nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0,
+                      "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS if ms > 0 else 0.0,
+                      "avg_ms": ms / max(cnt, 1), "algorithmic_GB_per_launch": nbytes / max(cnt, 1) / 1e9}
+
+    # ---- per shape, and bf16 nn.Linear on the same GPU
+    per_shape = {}
+    for lay in layers:
+        name = lay[0]
+        t = timed(torch, lambda: step([lay]), max(2, args.steps // 2), 1)
+        per_shape[name] = {"fp8_ms": t * 1e3, "fp8_TFLOP/s": flop_per_shape[name] / t / 1e12}
+    bf16_step = None
+    if not args.no_bf16:
+        for lay in layers:
+            name = lay[0]
+            t = timed(torch, lambda: step([lay], use_fp8=False), max(2, args.steps // 2), 1)
+            per_shape[name]["bf16_ms"] = t * 1e3
+            per_shape[name]["bf16_TFLOP/s"] = flop_per_shape[name] / t / 1e12
+            per_shape[name]["speedup_vs_bf16"] = per_shape[name]["bf16_ms"] / per_shape[name]["fp8_ms"]
+        bf16_step = sum(v["bf16_ms"] for v in per_shape.values()) * 1e-3
+
+    out = {
+        "metric": "Float8Linear fwd+bwd TFLOP/s at LLaMa-2-70B shapes (1 GPU); cast GB/s",
+        "value": flop_step / sec_step / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec_step * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8",
+        "data": "synthetic",
+        "config": {
+            "workload": f"LLaMa-2-70B linear shapes, dynamic scaling, M={m} tokens bf16, (K->N) 8192->10240, 8192->8192, "
+                        "8192->57344, 28672->8192; fwd+bwd with dY ~N(0,1e-2); one step = all four shapes",
+            "flop_per_step": flop_step,
+            "flop_convention": "3 * 2*M*K*N per shape",
+        },
+        "roofline": {
+            "kernel": "f8mi gemm_nt_kernel (fp8 MFMA GEMM, all 12 launches of a step)",
+            "bound": "mfma",
+            "achieved": gemm_tflops,
+            "peak": PEAK_FP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": gemm_tflops / PEAK_FP8_TFLOPS,
+            "traffic": None,
+            "launches": n_gemm,
+            "avg_launch_ms": ms_gemm / max(n_gemm, 1),
+            "flop_per_launch": flop_gemm / max(n_gemm, 1),
+        },
+        "hbm_kernels": hbm,
+        "per_shape": per_shape,
+        "frac_of_fp8_peak_end_to_end": flop_step / sec_step / 1e12 / PEAK_FP8_TFLOPS,
+    }
+    if bf16_step:
+        out["bf16_linear"] = {"ms_per_step": bf16_step * 1e3, "TFLOP/s": flop_step / bf16_step / 1e12,
+                              "speedup_fp8_over_bf16": bf16_step / sum(v["fp8_ms"] * 1e-3 for v in per_shape.values())}
+    if not args.no_cpu_baseline:
+        # free the GPU-side tensors' host shadows are none; the CPU leg only needs host memory
+        out["cpu_baseline"] = cpu_baseline(torch, args.cpu_seconds)
+        out["cpu_baseline"]["host"] = {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
+                                       "torch": torch.__version__}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

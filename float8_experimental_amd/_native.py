@@ -215,7 +215,7 @@ def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: t
         if t.shape[1] <= 1 or t.stride(1) == 1:
             if t.shape[0] <= 1 or t.stride(0) >= max(t.shape[1], 1):
                 return t, (t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1))
-        t = t.contiguous()
+        t = t.view(torch.uint8).contiguous().view(t.dtype)  # byte copy: not every fp8 dtype has copy kernels
         return t, max(t.shape[1], 1)
 
     a, lda = rowmajor(a)

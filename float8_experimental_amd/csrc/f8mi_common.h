@@ -49,7 +49,13 @@ __device__ __forceinline__ float fp16_bits_to_float(uint32_t h) {
     return __half2float(__ushort_as_half((unsigned short)h));
 }
 
-__device__ __forceinline__ float round_to_fp16(float f) { return __half2float(__float2half_rn(f)); }
+// fp32 -> fp16 -> fp32.  The empty asm pins `f` as a rounded fp32 value first: without it
+// the compiler folds a preceding multiply into one mixed-precision fma (single rounding,
+// and +0 addend, which turns -0 into +0), while the reference rounds twice.
+__device__ __forceinline__ float round_to_fp16(float f) {
+    asm volatile("" : "+v"(f));
+    return __half2float(__float2half_rn(f));
+}
 
 template <int DT>
 __device__ __forceinline__ float round_to(float f) {
@@ -86,12 +92,18 @@ __device__ __forceinline__ float amax_to_scale_dev(float amax, int math_dt, int 
 
 // Two fp32 -> two OCP fp8 bytes (low 16 bits of the result), round to nearest
 // even via the gfx950 conversion instructions.  Inputs must already be clamped
-// to the finite range or be NaN; NaN gives a NaN code.
+// to the finite range or be NaN.  NaN gives 0x7F (sign kept): the e4m3fn
+// instruction does that by itself, the e5m2 one returns the quiet-NaN code 0x7E,
+// so the low mantissa bit is set by hand to match torch's 0x7F.
 template <int FMT>
 __device__ __forceinline__ uint32_t cvt2_fp8(float a, float b) {
     uint32_t r;
-    if constexpr (FMT == F8MI_E4M3FN) r = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-    else r = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    if constexpr (FMT == F8MI_E4M3FN) {
+        r = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    } else {
+        r = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+        r |= (a != a ? 0x0001u : 0u) | (b != b ? 0x0100u : 0u);
+    }
     return r & 0xffffu;
 }
 

@@ -1,0 +1,127 @@
+"""Module swap and delayed-scaling bookkeeping (mirror of the reference's ``float8_linear_utils.py``)."""
+import logging
+from typing import Callable, List, Optional
+
+import torch
+import torch.nn as nn
+
+from . import _native
+from .config import Float8LinearConfig, ScalingType
+from .float8_linear import Float8Linear
+from .float8_utils import e4m3_dtype, e5m2_dtype
+
+log = logging.getLogger(__name__)
+log.addHandler(logging.NullHandler())
+
+_KINDS = (("input", e4m3_dtype), ("weight", e4m3_dtype), ("grad_output", e5m2_dtype))
+
+
+def linear_requires_sync(config: Float8LinearConfig) -> bool:
+    """True when any of the three tensors uses delayed scaling (reference :26-34)."""
+    return ScalingType.DELAYED in (config.cast_config_input.scaling_type, config.cast_config_weight.scaling_type,
+                                   config.cast_config_grad_output.scaling_type)
+
+
+def _update_history_stack(new_amax: torch.Tensor, amax_history_stack: torch.Tensor) -> torch.Tensor:
+    """Shifts every row of ``amax_history_stack`` [n, H] right by one and puts ``new_amax`` [n, 1]
+    in column 0, in place (reference :37-56)."""
+    assert amax_history_stack.dim() == 2, f"Expected amat_history_stack to be 2D, got {amax_history_stack.shape}"
+    assert new_amax.size(0) == amax_history_stack.size(0), (
+        f"Expected new_amax to have the same size as the first dimension of amax_history_stack, got "
+        f"{new_amax.size(0)} and {amax_history_stack.size(0)}")
+    shifted = torch.roll(amax_history_stack, 1, dims=1)
+    shifted[:, 0] = new_amax.squeeze(-1)
+    amax_history_stack.copy_(shifted)
+
+
+def swap_linear_layers(module: nn.Module, from_float_func: Callable[[nn.Linear], nn.Linear], *,
+                       module_filter_fn: Optional[Callable[[nn.Module, str], bool]] = None) -> nn.Module:
+    """Replaces every ``nn.Linear`` that passes ``module_filter_fn(module, fqn)`` by
+    ``from_float_func(module)`` (reference :59-122).  A root-level ``nn.Linear`` cannot be replaced
+    in place and is returned converted instead; children are visited before their parents."""
+    wanted = lambda m, fqn: isinstance(m, nn.Linear) and (module_filter_fn is None or module_filter_fn(m, fqn))
+    if wanted(module, ""):
+        if len(list(module.children())) > 0:
+            raise AssertionError(f"Does not support a root nn.Linear with children: {module}")
+        return from_float_func(module)
+
+    def visit(mod: nn.Module, fqn: str, parent: Optional[nn.Module], name: str):
+        for child_name, child in list(mod.named_children()):
+            visit(child, child_name if fqn == "" else f"{fqn}.{child_name}", mod, child_name)
+        if wanted(mod, fqn):
+            assert parent is not None, f"Linear root module should return early: {mod}"
+            setattr(parent, name, from_float_func(mod))
+
+    visit(module, "", None, "")
+    return module
+
+
+def convert_to_float8_training(module: nn.Module, *, module_filter_fn: Optional[Callable[[nn.Module, str], bool]] = None,
+                               config: Float8LinearConfig = None) -> nn.Module:
+    """Swaps ``nn.Linear`` modules for ``Float8Linear`` (reference :125-154)."""
+    if config is None:
+        config = Float8LinearConfig()
+    return swap_linear_layers(module, lambda m: Float8Linear.from_float(m, config=config),
+                              module_filter_fn=module_filter_fn)
+
+
+def get_float8_layers(model: torch.nn.Module) -> List[Float8Linear]:
+    """All Float8Linear modules of ``model`` (reference :157-169)."""
+    return [m for m in model.modules() if isinstance(m, Float8Linear)]
+
+
+_sync_tables = {}
+
+
+def _sync_table(fp8_layers) -> torch.Tensor:
+    """Device table of (amax, history, scale, format) pointers for all 3L buffers, rebuilt only when a
+    buffer has moved (``.to()``, ``load_state_dict`` into new storage, ...)."""
+    bufs = []
+    for child in fp8_layers:
+        for kind, f8 in _KINDS:
+            bufs.append((getattr(child, f"fp8_amax_{kind}"), getattr(child, f"fp8_amax_history_{kind}"),
+                         getattr(child, f"fp8_scale_{kind}"), f8))
+    key = tuple(t.data_ptr() for row in bufs for t in row[:3])
+    hit = _sync_tables.get(key)
+    if hit is None:
+        if len(_sync_tables) > 64:
+            _sync_tables.clear()
+        hit = _native.sync_table(bufs, bufs[0][0].device)
+        _sync_tables[key] = hit
+    return hit
+
+
+@torch.no_grad()
+def sync_float8_amax_and_scale_history(model: torch.nn.Module, fp8_layers=None) -> None:
+    """Turns the amaxes recorded during the last iteration into the scales of the next one and marks
+    the layers synced (reference :172-327).
+
+    For every layer and each of input / weight / grad_output:
+    ``S = roll(history, 1); S[0] = amax; scale = fmax / max(S)`` (fp32, two roundings).  Like the
+    reference -- which rolls a stacked copy and copies only the scales back (:287-319) -- the
+    layers' history buffers themselves are left as they are.  All of it is one kernel launch.
+    The MAX all-reduce of the amaxes over ranks (:261-284) needs more than one GPU.
+    """
+    if fp8_layers is None:
+        fp8_layers = get_float8_layers(model)
+    if len(fp8_layers) == 0:
+        log.warning("Calling sync_float8_amax_and_scale_history on a module with no Float8Linear layers")
+        return
+
+    x_dtypes = {child.last_seen_input_dtype for child in fp8_layers}
+    if len(x_dtypes) != 1:
+        raise ValueError(f"All layers must have the same last seen input_dtype, got {x_dtypes}")
+    recipes = {child.config.delayed_scaling_config.scale_fn_name for child in fp8_layers}
+    if len(recipes) != 1:
+        raise ValueError(f"All layers must have the same scale_fn recipe, got {recipes}")
+    hist_lens = {child.config.delayed_scaling_config.history_len for child in fp8_layers}
+    if len(hist_lens) != 1:
+        raise ValueError(f"All layers must have the same history_len, got {hist_lens}")
+    if torch.distributed.is_available() and torch.distributed.is_initialized() and torch.distributed.get_world_size() > 1:
+        raise NotImplementedError("amax all-reduce across ranks: this build drives a single GPU")
+
+    table = _sync_table(fp8_layers)
+    _native.sync(table, next(iter(hist_lens)), next(iter(x_dtypes)) is torch.float16, writeback_history=False)
+
+    for child in fp8_layers:
+        child.amax_and_scale_synced = True

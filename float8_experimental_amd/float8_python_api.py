@@ -1,0 +1,27 @@
+"""``addmm_float8_unwrapped``: the scaled fp8 matmul on plain tensors
+(mirror of the reference's ``float8_python_api.py``, which forwards to ``torch._scaled_mm``).
+"""
+from typing import Optional
+
+import torch
+
+from . import _native
+
+
+def addmm_float8_unwrapped(a_data: torch.Tensor, a_scale: torch.Tensor, b_data: torch.Tensor, b_scale: torch.Tensor,
+                           output_dtype: torch.dtype, output_scale: Optional[torch.Tensor] = None,
+                           bias: Optional[torch.Tensor] = None, use_fast_accum: bool = False) -> torch.Tensor:
+    """``(a_data @ b_data) / (a_scale * b_scale) (+ bias)`` on the gfx950 matrix cores.
+
+    ``a_data`` is fp8 ``[m, k]``, ``b_data`` fp8 ``[k, n]``; as in the reference
+    (float8_python_api.py:24-64) the scales are the tensors' forward scales and the
+    kernel applies their reciprocals.  The kernel wants both operands contiguous along
+    k: ``a_data`` row-major and ``b_data`` column-major pass through untouched (the
+    layout float8_ops.preprocess_addmm guarantees), anything else is copied once.
+    ``use_fast_accum`` has no effect on this hardware.  ``output_scale`` (fp8 output) is
+    not implemented, as in the reference's own call sites, which always pass None.
+    """
+    if output_scale is not None:
+        raise NotImplementedError("fp8 output of the scaled matmul is not supported")
+    assert a_data.dim() == 2 and b_data.dim() == 2 and a_data.shape[1] == b_data.shape[0]
+    return _native.gemm_nt(a_data, a_scale, b_data.t(), b_scale, output_dtype, bias=bias)
