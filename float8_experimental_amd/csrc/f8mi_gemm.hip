@@ -3,14 +3,29 @@
 //
 // Workgroup = 256 lanes (4 waves, 2 x 2), macro tile 256 x 256, K step 128 bytes.
 // Each wave owns 128 x 128 of C = 4 x 4 MFMA tiles of 32 x 32 (256 accumulator
-// registers).  Operand tiles are staged HBM -> registers -> LDS (two stages, 64 KB
-// each) as 16-byte pieces; piece c of tile row r lives at r*128 + ((c ^ (r & 7)) * 16),
-// which makes both the 16-byte LDS writes and the per-lane 2 x 16-byte fragment
-// reads (lane = tile row, 32 consecutive k per lane) bank-conflict free.
+// registers), so there is one wave per SIMD and nothing hides latency for it:
+// the loop is software-pipelined by hand.
+//   * HBM -> registers -> LDS, two LDS stages of 64 KB.  The loads of K step
+//     kb+2 are in flight while step kb is multiplied; they are written to the
+//     free stage one iteration later, in small groups between MFMAs.
+//   * LDS -> registers: every lane needs 32 consecutive k of one tile row per
+//     MFMA (2 x 16-byte reads).  Fragments are double-buffered in registers: the
+//     reads for the next 64-deep half step are issued between the MFMAs of the
+//     current one.
+//   * 16-byte piece c of tile row r lives at r*128 + ((c ^ ((r >> 1) & 7)) * 16): the
+//     fragment reads run at the LDS's full 256 bytes per clock (64 banks).
+//   * one s_barrier per K step, waiting on LDS traffic only (never on the HBM
+//     loads in flight).
+// The MFMA is issued with the Bt rows as its first operand, so a lane ends up
+// holding 4 consecutive columns of one row of C: the epilogue scales, converts
+// (v_cvt_pk_bf16_f32), packs 8 bytes per lane into a padded LDS tile and writes C
+// with 16-byte stores, 256 contiguous bytes per row and wave.
 // Workgroup ids are first re-dealt so that each of the 8 XCDs (which receive
 // consecutive ids round-robin) works on one contiguous band of tiles, then
 // walked in groups of 8 tile rows so the tiles in flight share A and B panels
 // in that XCD's L2.
+#include <type_traits>
+
 #include "f8mi_common.h"
 
 namespace f8mi {
@@ -21,9 +36,16 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int BM = 256, BN = 256, BK = 128;
 constexpr int GEMM_THREADS = 256;
 constexpr int STAGE_BYTES = (BM + BN) * BK;  // 64 KB
-constexpr int GEMM_LDS = 2 * STAGE_BYTES;    // 128 KB
+constexpr int EPI_PITCH = 128 * 2 + 16;      // bytes per row of a wave's 128 x 128 2-byte output tile in LDS
+constexpr int EPI_BYTES = 4 * 128 * EPI_PITCH;
+constexpr int GEMM_LDS = 2 * STAGE_BYTES > EPI_BYTES ? 2 * STAGE_BYTES : EPI_BYTES;
 constexpr int GROUP_M = 8;
 constexpr int NUM_XCD = 8;
+
+#define F8MI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Workgroup barrier that waits for this wave's LDS traffic only.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // 16 bytes of one operand row; bytes at k >= klimit read as zero.
 template <bool ALIGNED, bool GUARD>
@@ -46,11 +68,37 @@ __device__ __forceinline__ uint4 load_piece(const uint8_t* __restrict__ p, int v
     return v;
 }
 
-template <int AF, int BF, bool ALIGNED>
+__device__ __forceinline__ v8i read_frag(const uint8_t* p0, const uint8_t* p1) {
+    const uint4 lo = *(const uint4*)p0;
+    const uint4 hi = *(const uint4*)p1;
+    return (v8i){(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+}
+
+template <int C_DT>
+__device__ __forceinline__ float load_bias(const void* bias, int col) {
+    if constexpr (C_DT == F8MI_BF16) return bf16_bits_to_float(((const uint16_t*)bias)[col]);
+    else if constexpr (C_DT == F8MI_FP16) return fp16_bits_to_float(((const uint16_t*)bias)[col]);
+    else return ((const float*)bias)[col];
+}
+
+// two fp32 -> two packed 2-byte outputs (round to nearest even)
+template <int C_DT>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    if constexpr (C_DT == F8MI_BF16) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        bf2 r = __builtin_convertvector((f2){a, b}, bf2);
+        return __builtin_bit_cast(uint32_t, r);
+    } else {
+        return (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+    }
+}
+
+template <int AF, int BF, bool ALIGNED, int C_DT>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_kernel(
     const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Bt, int64_t ldb, int M, int N, int K,
-    const float* __restrict__ sa_dev, const float* __restrict__ sb_dev, void* __restrict__ C, int c_dtype,
-    int64_t ldc, const void* __restrict__ bias, int tiles_m, int tiles_n) {
+    const float* __restrict__ sa_dev, const float* __restrict__ sb_dev, void* __restrict__ C, int64_t ldc,
+    const void* __restrict__ bias, int tiles_m, int tiles_n, int c_vec_ok) {
     extern __shared__ __align__(16) uint8_t smem[];
 
     // ---- which tile
@@ -69,50 +117,52 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_kernel(
     const int lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
-    // ---- global -> register staging: piece (row = i*32 + t/8, c = t%8), i = 0..7, per operand
-    const int lrow = t >> 3, lc = t & 7;
+    // ---- global -> register staging.  Lane t moves, per operand, rows i*64 + t/4 (i = 0..3) and of each
+    // row the 16-byte pieces t%4 (first 64-deep half step) and t%4 + 4 (second half step).
+    const int lrow = t >> 2, lc = t & 3;
     const uint8_t* a_base = A + (int64_t)m0 * lda;
     const uint8_t* b_base = Bt + (int64_t)n0 * ldb;
-    uint32_t a_off[8], b_off[8];
+    uint32_t a_off[4], b_off[4];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int r = i * 32 + lrow;
+    for (int i = 0; i < 4; i++) {
+        const int r = i * 64 + lrow;
         a_off[i] = (uint32_t)(min(r, M - 1 - m0) * lda) + lc * 16;  // rows past the edge re-read the last row
         b_off[i] = (uint32_t)(min(r, N - 1 - n0) * ldb) + lc * 16;
     }
-    const int st_off = lrow * BK + ((lc ^ (lrow & 7)) << 4);  // + i*32*BK
+    // piece c of tile row r sits at r*128 + ((c ^ swz(r)) * 16), swz(r) = (r >> 1) & 7: the LDS has 64
+    // banks (256 bytes per clock), so the 16 lanes served together by a 16-byte read -- 16 consecutive
+    // rows, same piece -- must land in 16 different 16-byte columns of a 256-byte span: the row parity
+    // picks the 128-byte half, the swizzle the column inside it
+    const int lsw = (lrow >> 1) & 7;
+    const int st_off0 = lrow * BK + ((lc ^ lsw) << 4);        // + i*64*BK, half step 0 piece
+    const int st_off1 = lrow * BK + (((lc + 4) ^ lsw) << 4);  // half step 1 piece
 
     const int nk_full = K / BK;
     const int nk = (K + BK - 1) / BK;
 
-    uint4 ra[8], rb[8];
-    auto gload = [&](int kb) {
-        const int k0 = kb * BK;
-        if (ALIGNED && kb < nk_full) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) ra[i] = load_piece<ALIGNED, false>(a_base + a_off[i] + k0, 16);
-#pragma unroll
-            for (int i = 0; i < 8; i++) rb[i] = load_piece<ALIGNED, false>(b_base + b_off[i] + k0, 16);
+    uint4 ra[4][2], rb[4][2];  // staging registers [row slot][half]
+    // GUARD = false: K step kb lies completely inside [0, K) and rows are 16-byte aligned
+    auto gload = [&](int kb, int i, int h, auto guard) __attribute__((always_inline)) {
+        const int k0 = kb * BK + h * 64;
+        const uint8_t* pa = a_base + k0;
+        const uint8_t* pb = b_base + k0;
+        if constexpr (!decltype(guard)::value) {
+            ra[i][h] = load_piece<ALIGNED, false>(pa + a_off[i], 16);
+            rb[i][h] = load_piece<ALIGNED, false>(pb + b_off[i], 16);
         } else {
-            const int valid = K - k0 - lc * 16;
-#pragma unroll
-            for (int i = 0; i < 8; i++) ra[i] = load_piece<ALIGNED, true>(a_base + a_off[i] + k0, valid);
-#pragma unroll
-            for (int i = 0; i < 8; i++) rb[i] = load_piece<ALIGNED, true>(b_base + b_off[i] + k0, valid);
+            ra[i][h] = load_piece<ALIGNED, true>(pa + a_off[i], K - k0 - lc * 16);
+            rb[i][h] = load_piece<ALIGNED, true>(pb + b_off[i], K - k0 - lc * 16);
         }
     };
-    auto lstore = [&](int stage) {
-        uint8_t* as = smem + stage * STAGE_BYTES;
-        uint8_t* bs = as + BM * BK;
-#pragma unroll
-        for (int i = 0; i < 8; i++) *(uint4*)(as + st_off + i * 32 * BK) = ra[i];
-#pragma unroll
-        for (int i = 0; i < 8; i++) *(uint4*)(bs + st_off + i * 32 * BK) = rb[i];
+    auto lstore = [&](uint8_t* stage, int i, int h) __attribute__((always_inline)) {
+        const int off = (h ? st_off1 : st_off0) + i * 64 * BK;
+        *(uint4*)(stage + off) = ra[i][h];
+        *(uint4*)(stage + BM * BK + off) = rb[i][h];
     };
 
     // ---- fragment addressing: lane -> tile row (lane % 32), k half (lane / 32)
     const int frow = lane & 31, fh = lane >> 5;
-    const int fsw = frow & 7;
+    const int fsw = (frow >> 1) & 7;
     int f_off[2][2];  // [ks][j]: byte offset of piece (ks*4 + fh*2 + j) of row frow
 #pragma unroll
     for (int ks = 0; ks < 2; ks++)
@@ -120,7 +170,15 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_kernel(
         for (int j = 0; j < 2; j++) f_off[ks][j] = frow * BK + (((ks * 4 + fh * 2 + j) ^ fsw) << 4);
     const int a_frag_base = (wm * 128) * BK;
     const int b_frag_base = BM * BK + (wn * 128) * BK;
+    auto frag_a = [&](const uint8_t* stage, int ks, int ti) __attribute__((always_inline)) {
+        return read_frag(stage + a_frag_base + ti * 32 * BK + f_off[ks][0], stage + a_frag_base + ti * 32 * BK + f_off[ks][1]);
+    };
+    auto frag_b = [&](const uint8_t* stage, int ks, int tj) __attribute__((always_inline)) {
+        return read_frag(stage + b_frag_base + tj * 32 * BK + f_off[ks][0], stage + b_frag_base + tj * 32 * BK + f_off[ks][1]);
+    };
 
+    // acc[tj][ti]: MFMA(first = Bt rows (n), second = A rows (m)) -> lane holds m = lane%32,
+    // n = 8*(e/4) + 4*(lane/32) + e%4 of its 32 x 32 tile
     v16f acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -129,89 +187,216 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_kernel(
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    if (nk > 0) {
-        gload(0);
-        lstore(0);
-        if (nk > 1) gload(1);
-    }
-    __syncthreads();
+    // Fragment registers.  The four Bt fragments of a half step are all live during it while the next
+    // half step's four are being fetched; the A fragment is needed one 4-MFMA group at a time.
+    v8i fb[2][4];  // [half-step parity][n tile]
+    v8i fa[2];     // rolling: group g multiplies fa[g & 1] while fa[(g + 1) & 1] is being fetched
 
-    for (int kb = 0; kb < nk; kb++) {
-        const uint8_t* st = smem + (kb & 1) * STAGE_BYTES;
+    constexpr std::true_type yes{};
+    constexpr std::false_type no{};
+
+    // Fills stage 0 with K step 0, starts the loads of K step 1 and fetches the first fragments.
+    // The loads of K step 1 are issued in the loop's own order (and pinned there) so that the
+    // compiler's count of loads in flight at the loop head is exact; a pessimistic count would make
+    // every iteration wait for loads it has only just issued.
+    auto prologue = [&](auto guard) __attribute__((always_inline)) {
+        constexpr bool G = decltype(guard)::value;
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-            v8i af[4], bf[4];
+        for (int i = 0; i < 4; i++) { gload(0, i, 0, guard); gload(0, i, 1, guard); }
 #pragma unroll
-            for (int ti = 0; ti < 4; ti++) {
-                const uint4 lo = *(const uint4*)(st + a_frag_base + ti * 32 * BK + f_off[ks][0]);
-                const uint4 hi = *(const uint4*)(st + a_frag_base + ti * 32 * BK + f_off[ks][1]);
-                af[ti] = (v8i){(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-            }
+        for (int i = 0; i < 4; i++) { lstore(smem, i, 0); lstore(smem, i, 1); }
+        if (!G || nk > 1) {
 #pragma unroll
-            for (int tj = 0; tj < 4; tj++) {
-                const uint4 lo = *(const uint4*)(st + b_frag_base + tj * 32 * BK + f_off[ks][0]);
-                const uint4 hi = *(const uint4*)(st + b_frag_base + tj * 32 * BK + f_off[ks][1]);
-                bf[tj] = (v8i){(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-            }
+            for (int h = 0; h < 2; h++)
 #pragma unroll
-            for (int ti = 0; ti < 4; ti++)
+                for (int i = 0; i < 4; i++) {
+                    F8MI_SCHED_FENCE();
+                    gload(1, i, h, guard);
+                }
+        }
+        F8MI_SCHED_FENCE();
+        lds_barrier();
+#pragma unroll
+        for (int x = 0; x < 4; x++) fb[0][x] = frag_b(smem, 0, x);
+        fa[0] = frag_a(smem, 0, 0);
+    };
+
+    // One K step = two half steps of 4 groups of 4 MFMAs.  Slotted in between the MFMAs, evenly spread:
+    // the fragment reads for the next group / half step, the 16-byte LDS writes of K step kb+1 (first
+    // its half-step-0 pieces, after the middle barrier its half-step-1 pieces) into the other stage, and
+    // the loads of K step kb+2 into the registers just written out.
+    // STEADY = true: K steps kb+1 and kb+2 exist and kb+2 needs no guards, so the body is
+    // straight-line code; the (at most three) last steps of a tile run the general version.
+    auto k_step = [&](int kb, auto steady) __attribute__((always_inline)) {
+        constexpr bool STEADY = decltype(steady)::value;
+        uint8_t* cur = smem + (kb & 1) * STAGE_BYTES;
+        uint8_t* nxt = smem + ((kb + 1) & 1) * STAGE_BYTES;
+        const bool has1 = STEADY || kb + 1 < nk, has2 = STEADY || kb + 2 < nk;
+
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                if (h == 0) {
+                    fa[(g + 1) & 1] = g < 3 ? frag_a(cur, 0, g + 1) : frag_a(cur, 1, 0);
+                    fb[1][g] = frag_b(cur, 1, g);
+                } else {
+                    if (g < 3) fa[(g + 1) & 1] = frag_a(cur, 1, g + 1);
+                    else if (has1) fa[0] = frag_a(nxt, 0, 0);
+                    if (has1) fb[0][g] = frag_b(nxt, 0, g);
+                }
+                if (has1) lstore(nxt, g, h);
+                if (has2) {
+                    if constexpr (STEADY) gload(kb + 2, g, h, no);
+                    else gload(kb + 2, g, h, yes);
+                }
 #pragma unroll
                 for (int tj = 0; tj < 4; tj++)
-                    acc[ti][tj] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[ti], bf[tj], acc[ti][tj], AF, BF,
-                                                                                 0, 0, 0, 0);
+                    acc[tj][g] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[h][tj], fa[g & 1], acc[tj][g], BF, AF, 0, 0, 0, 0);
+                // A wave cannot run ahead of an MFMA it has not issued yet, so everything else has to be
+                // slotted in between the MFMAs (each keeps the matrix core busy for 64 cycles) rather than
+                // after them: MFMA, 2 LDS reads, MFMA, LDS write + load, twice.
+#pragma unroll
+                for (int rep = 0; rep < 2; rep++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS read
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS write
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global load
+                }
+                F8MI_SCHED_FENCE();
+            }
+            // h = 0: the half-step-0 pieces of K step kb+1 are in place for everybody;
+            // h = 1: its half-step-1 pieces are, and every wave is done reading `cur`.
+            lds_barrier();
         }
-        if (kb + 1 < nk) {
-            lstore((kb + 1) & 1);
-            if (kb + 2 < nk) gload(kb + 2);
-        }
-        __syncthreads();
+    };
+
+    const int n_steady = ALIGNED ? max(nk_full - 2, 0) : 0;
+    if (n_steady > 0) {  // at least three full, aligned K steps
+        prologue(no);
+        int kb = 0;
+        for (; kb < n_steady; kb++) k_step(kb, yes);
+        for (; kb < nk; kb++) k_step(kb, no);
+    } else if (nk > 0) {
+        prologue(yes);
+        for (int kb = 0; kb < nk; kb++) k_step(kb, no);
     }
 
-    // ---- epilogue: scale, (+bias), convert, store.  acc[ti][tj][e] of lane l is
-    // C[row = 8*(e/4) + 4*(l/32) + e%4][col = l%32] of its 32 x 32 tile.
+    // ---- epilogue
     const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
-#pragma unroll
-    for (int tj = 0; tj < 4; tj++) {
-        const int col = n0 + wn * 128 + tj * 32 + (lane & 31);
-        if (col >= N) continue;
-        float bv = 0.0f;
-        if (bias) {
-            if (c_dtype == F8MI_BF16) bv = bf16_bits_to_float(((const uint16_t*)bias)[col]);
-            else if (c_dtype == F8MI_FP16) bv = fp16_bits_to_float(((const uint16_t*)bias)[col]);
-            else bv = ((const float*)bias)[col];
-        }
+    const int lm = lane & 31, lh = lane >> 5;
+    const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
+
+    if constexpr (C_DT == F8MI_FP32) {
+        // 4 consecutive columns per lane = one 16-byte store
+        float* Cf = (float*)C;
 #pragma unroll
         for (int ti = 0; ti < 4; ti++) {
+            const int row = wrow0 + ti * 32 + lm;
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int row = m0 + wm * 128 + ti * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (row >= M) continue;
-                const float v = acc[ti][tj][e] * inv + bv;
-                const int64_t idx = (int64_t)row * ldc + col;
-                if (c_dtype == F8MI_BF16) ((uint16_t*)C)[idx] = (uint16_t)float_to_bf16_bits(v);
-                else if (c_dtype == F8MI_FP16) ((__half*)C)[idx] = __float2half_rn(v);
-                else ((float*)C)[idx] = v;
+            for (int tj = 0; tj < 4; tj++) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int col = wcol0 + tj * 32 + 8 * g + 4 * lh;
+                    if (row >= M || col >= N) continue;
+                    float v[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        v[r] = acc[tj][ti][4 * g + r] * inv;
+                        if (bias && col + r < N) v[r] += load_bias<C_DT>(bias, col + r);
+                    }
+                    float* dst = Cf + (int64_t)row * ldc + col;
+                    if (c_vec_ok && col + 4 <= N) {
+                        *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (col + r < N) dst[r] = v[r];
+                    }
+                }
+            }
+        }
+    } else {
+        // all waves are done with the operand stages before they become the output staging area
+        lds_barrier();
+        uint8_t* ep = smem + wave * (128 * EPI_PITCH);
+#pragma unroll
+        for (int tj = 0; tj < 4; tj++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int cl = tj * 32 + 8 * g + 4 * lh;  // column inside the wave's 128
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (bias) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (wcol0 + cl + r < N) bv[r] = load_bias<C_DT>(bias, wcol0 + cl + r);
+                }
+#pragma unroll
+                for (int ti = 0; ti < 4; ti++) {
+                    const float v0 = acc[tj][ti][4 * g + 0] * inv + bv[0];
+                    const float v1 = acc[tj][ti][4 * g + 1] * inv + bv[1];
+                    const float v2 = acc[tj][ti][4 * g + 2] * inv + bv[2];
+                    const float v3 = acc[tj][ti][4 * g + 3] * inv + bv[3];
+                    *(uint2*)(ep + (ti * 32 + lm) * EPI_PITCH + cl * 2) = make_uint2(pack2<C_DT>(v0, v1), pack2<C_DT>(v2, v3));
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own wave's tile only: no workgroup barrier needed
+        uint16_t* Ch = (uint16_t*)C;
+        const int chunk = lane & 15, rsub = lane >> 4;
+        const int col = wcol0 + chunk * 8;
+#pragma unroll 4
+        for (int it = 0; it < 32; it++) {
+            const int rl = it * 4 + rsub;
+            const int row = wrow0 + rl;
+            const uint4 v = *(const uint4*)(ep + rl * EPI_PITCH + chunk * 16);
+            if (row < M && col < N) {
+                uint16_t* dst = Ch + (int64_t)row * ldc + col;
+                if (c_vec_ok && col + 8 <= N) {
+                    *(uint4*)dst = v;
+                } else {
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++)
+                        if (col + i < N) dst[i] = (uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+                }
             }
         }
     }
 }
 
-template <int AF, int BF>
-static int launch_gemm(bool aligned, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, const uint8_t* Bt,
-                       int64_t ldb, int M, int N, int K, const float* sa, const float* sb, void* C, int c_dtype,
-                       int64_t ldc, const void* bias, int tiles_m, int tiles_n) {
-    static bool attr_done[2] = {false, false};
-    auto ka = gemm_nt_kernel<AF, BF, true>;
-    auto ku = gemm_nt_kernel<AF, BF, false>;
-    if (!attr_done[aligned ? 1 : 0]) {
-        hipError_t e = hipFuncSetAttribute(aligned ? (const void*)ka : (const void*)ku,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
+template <int AF, int BF, bool ALIGNED, int C_DT>
+static int launch_gemm3(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, const uint8_t* Bt, int64_t ldb, int M,
+                        int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
+                        int tiles_m, int tiles_n, int c_vec_ok) {
+    static bool attr_done = false;
+    auto kern = gemm_nt_kernel<AF, BF, ALIGNED, C_DT>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
         if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-        attr_done[aligned ? 1 : 0] = true;
+        attr_done = true;
     }
-    if (aligned) hipLaunchKernelGGL(ka, g, dim3(GEMM_THREADS), GEMM_LDS, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, c_dtype, ldc, bias, tiles_m, tiles_n);
-    else hipLaunchKernelGGL(ku, g, dim3(GEMM_THREADS), GEMM_LDS, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, c_dtype, ldc, bias, tiles_m, tiles_n);
+    hipLaunchKernelGGL(kern, g, dim3(GEMM_THREADS), GEMM_LDS, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias,
+                       tiles_m, tiles_n, c_vec_ok);
     return check_hip(hipGetLastError(), "gemm kernel launch");
+}
+
+template <int AF, int BF, bool ALIGNED>
+static int launch_gemm2(int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, const uint8_t* Bt,
+                        int64_t ldb, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
+                        const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    if (c_dtype == F8MI_BF16) return launch_gemm3<AF, BF, ALIGNED, F8MI_BF16>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (c_dtype == F8MI_FP16) return launch_gemm3<AF, BF, ALIGNED, F8MI_FP16>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch_gemm3<AF, BF, ALIGNED, F8MI_FP32>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+}
+
+template <int AF, int BF>
+static int launch_gemm1(bool aligned, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda,
+                        const uint8_t* Bt, int64_t ldb, int M, int N, int K, const float* sa, const float* sb, void* C,
+                        int64_t ldc, const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    if (aligned) return launch_gemm2<AF, BF, true>(c_dtype, g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch_gemm2<AF, BF, false>(c_dtype, g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
 }
 
 }  // namespace f8mi
@@ -232,13 +417,15 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7fffffff) { set_error("f8mi_gemm_nt: too many tiles"); return F8MI_ERR_UNSUPPORTED; }
     const bool aligned = ((uintptr_t)a % 16 == 0) && ((uintptr_t)bt % 16 == 0) && (lda % 16 == 0) && (ldb % 16 == 0);
+    const int64_t csz = c_dtype == F8MI_FP32 ? 4 : 2;
+    const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
     const uint8_t* A = (const uint8_t*)a;
     const uint8_t* B = (const uint8_t*)bt;
     const int M = (int)m, N = (int)n, K = (int)k;
-    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_gemm<0, 0>(aligned, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, (int)tiles_m, (int)tiles_n);
-    if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_gemm<1, 0>(aligned, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, (int)tiles_m, (int)tiles_n);
-    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_gemm<0, 1>(aligned, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, (int)tiles_m, (int)tiles_n);
-    return launch_gemm<1, 1>(aligned, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, (int)tiles_m, (int)tiles_n);
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_gemm1<0, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_gemm1<1, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_gemm1<0, 1>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    return launch_gemm1<1, 1>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
 }
