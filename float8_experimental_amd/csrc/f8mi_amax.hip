@@ -11,7 +11,7 @@
 namespace f8mi {
 
 constexpr int AMAX_THREADS = 256;
-constexpr int AMAX_UNROLL = 4;  // 16-byte loads in flight per thread
+constexpr int AMAX_UNROLL = 8;  // 16-byte loads in flight per thread
 
 // sign-cleared patterns of the elements packed in one 32-bit word, reduced to one value
 template <int DT>
@@ -56,7 +56,9 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* lds) {
 __device__ __forceinline__ void publish_amax(uint32_t blockmax, uint32_t* ws, float* amax_out, float* scale_out,
                                              int in_dt, int math_dt, int fmt, int orig_is_fp16) {
     if (threadIdx.x == 0) {
-        if (blockmax) atomicMax(&ws[WS_AMAX_BITS], blockmax);
+        // the running maximum only grows: a (possibly stale) read that is already >= this block's value
+        // makes the atomic unnecessary, which keeps thousands of blocks from queueing on one address
+        if (blockmax > __atomic_load_n(&ws[WS_AMAX_BITS], __ATOMIC_RELAXED)) atomicMax(&ws[WS_AMAX_BITS], blockmax);
         __threadfence();
         uint32_t ticket = atomicAdd(&ws[WS_TICKET], 1u);
         if (ticket == gridDim.x * gridDim.y - 1) {
@@ -70,26 +72,37 @@ __device__ __forceinline__ void publish_amax(uint32_t blockmax, uint32_t* ws, fl
     }
 }
 
-// x is dense (ld == cols) and 16-byte aligned: 1-D grid-stride over 16-byte vectors.
+// x is dense (ld == cols) and 16-byte aligned.  A block walks over tiles of AMAX_THREADS * AMAX_UNROLL
+// 16-byte vectors (32 KB of contiguous memory); inside a tile consecutive lanes read consecutive
+// vectors, so every wave-level load is 1 KB of one DRAM page.  (Striding each lane's loads by the whole
+// grid instead costs more than half of the bandwidth.)
 template <int DT>
 __global__ __launch_bounds__(AMAX_THREADS) void amax_dense_kernel(const void* __restrict__ x, int64_t n,
                                                                    uint32_t* ws, float* amax_out, float* scale_out,
                                                                    int math_dt, int fmt, int orig_is_fp16) {
     __shared__ uint32_t red[AMAX_THREADS / 64];
     constexpr int EPV = DT == F8MI_FP32 ? 4 : 8;
+    constexpr int64_t TILE = (int64_t)AMAX_THREADS * AMAX_UNROLL;
     const int64_t nvec = n / EPV;
     const uint4* xv = (const uint4*)x;
     uint32_t m = 0;
-    const int64_t stride = (int64_t)gridDim.x * AMAX_THREADS;
-    int64_t i = (int64_t)blockIdx.x * AMAX_THREADS + threadIdx.x;
-    for (; i + (AMAX_UNROLL - 1) * stride < nvec; i += AMAX_UNROLL * stride) {
+    const int64_t ntiles = (nvec + TILE - 1) / TILE;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const int64_t base = t * TILE + threadIdx.x;
         uint4 v[AMAX_UNROLL];
+        if (base - threadIdx.x + TILE <= nvec) {
 #pragma unroll
-        for (int u = 0; u < AMAX_UNROLL; u++) v[u] = load_nt16(&xv[i + u * stride]);
+            for (int u = 0; u < AMAX_UNROLL; u++) v[u] = load_nt16(&xv[base + u * AMAX_THREADS]);
+        } else {
+#pragma unroll
+            for (int u = 0; u < AMAX_UNROLL; u++) {
+                const int64_t i = base + u * AMAX_THREADS;
+                v[u] = i < nvec ? load_nt16(&xv[i]) : make_uint4(0, 0, 0, 0);
+            }
+        }
 #pragma unroll
         for (int u = 0; u < AMAX_UNROLL; u++) m = absmax_vec<DT>(v[u], m);
     }
-    for (; i < nvec; i += stride) m = absmax_vec<DT>(load_nt16(&xv[i]), m);
     if (blockIdx.x == 0) {  // scalar tail (< EPV elements)
         int64_t t = nvec * EPV + threadIdx.x;
         if (t < n) {
@@ -167,7 +180,7 @@ extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_
         const int64_t epv = 16 / esz;
         const int64_t nvec = n / epv;
         int64_t blocks = (nvec + (int64_t)AMAX_THREADS * AMAX_UNROLL - 1) / ((int64_t)AMAX_THREADS * AMAX_UNROLL);
-        const int64_t cap = (int64_t)cu_count() * 8;
+        const int64_t cap = (int64_t)cu_count() * 2;  // few, long-lived blocks: one ticket atomic each
         if (blocks > cap) blocks = cap;
         if (blocks < 1) blocks = 1;
         dim3 g((unsigned)blocks), b(AMAX_THREADS);

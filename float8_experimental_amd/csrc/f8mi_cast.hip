@@ -18,32 +18,40 @@ namespace f8mi {
 
 constexpr int CAST_THREADS = 256;
 constexpr int CAST_TILE = 128;
+constexpr int CAST_GROUP = 8;
 
-__device__ __forceinline__ void publish_amax_cast(uint32_t blockmax, uint32_t* ws, float* amax_out, int in_dt) {
+// Fused amax of the cast kernel: *amax_out was zeroed by a tiny kernel launched just before, and holds the
+// running maximum as an fp32 bit pattern (non-negative floats and NaNs order like unsigned integers).
+// No ticket and, for all but a handful of blocks, no atomic at all: the value only grows, so a block whose
+// maximum is not above a (possibly stale) read of it has nothing to add.
+__device__ __forceinline__ void publish_amax_cast(uint32_t blockmax, float* amax_out, int in_dt) {
     if (threadIdx.x == 0) {
-        if (blockmax) atomicMax(&ws[WS_AMAX_BITS], blockmax);
-        __threadfence();
-        uint32_t ticket = atomicAdd(&ws[WS_TICKET], 1u);
-        if (ticket == gridDim.x * gridDim.y - 1) {
-            __threadfence();
-            uint32_t bits = atomicExch(&ws[WS_AMAX_BITS], 0u);
-            atomicExch(&ws[WS_TICKET], 0u);
-            *amax_out = abs_bits_to_float(bits, in_dt);
-        }
+        const uint32_t bits = __float_as_uint(abs_bits_to_float(blockmax, in_dt));
+        uint32_t* dst = (uint32_t*)amax_out;
+        if (bits > __atomic_load_n(dst, __ATOMIC_RELAXED)) atomicMax(dst, bits);
     }
 }
 
-// One element: x*scale rounded to PROD, clamped (NaN kept), as fp32 ready for conversion.
-template <int PROD>
-__device__ __forceinline__ float scale_clamp(float x, float scale, float fmax) {
-    float y = round_to<PROD>(__fmul_rn(x, scale));
-    float c = fminf(fmaxf(y, -fmax), fmax);  // drops NaN ...
-    return (y != y) ? y : c;                 // ... so put it back
+// clamp to [-fmax, fmax], NaN kept (v_med3_f32 drops it, so it is put back)
+__device__ __forceinline__ float clamp_keep_nan(float y, float fmax) {
+    const float c = __builtin_amdgcn_fmed3f(y, -fmax, fmax);
+    return (y != y) ? y : c;
 }
 
-template <int FMT>
-__device__ __forceinline__ uint32_t pack4(float a, float b, float c, float d) {
-    return cvt2_fp8<FMT>(a, b) | (cvt2_fp8<FMT>(c, d) << 16);
+// Two adjacent elements: x*scale rounded to PROD, clamped, as fp32 ready for conversion.
+template <int PROD>
+__device__ __forceinline__ void scale_clamp2(float x0, float x1, float scale, float fmax, float& y0, float& y1) {
+    float p0 = __fmul_rn(x0, scale), p1 = __fmul_rn(x1, scale);
+    if constexpr (PROD == F8MI_BF16) {
+        const uint32_t w = pack_bf16x2(p0, p1);
+        p0 = __uint_as_float(w << 16);
+        p1 = __uint_as_float(w & 0xffff0000u);
+    } else if constexpr (PROD == F8MI_FP16) {
+        p0 = round_to_fp16(p0);
+        p1 = round_to_fp16(p1);
+    }
+    y0 = clamp_keep_nan(p0, fmax);
+    y1 = clamp_keep_nan(p1, fmax);
 }
 
 // 4 dwords (rows 0..3, 4 bytes each = columns 0..3) -> 4 dwords (column c: rows 0..3)
@@ -124,15 +132,34 @@ template <int DT, int PROD, int FMT, bool VEC>
 __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
                                                             int64_t ld, const float* __restrict__ scale_dev,
                                                             uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
-                                                            float* amax_out, uint32_t* ws) {
+                                                            float* amax_out, int64_t tiles_x, int64_t tiles_y) {
     __shared__ uint32_t tileT[CAST_TILE * CAST_TILE / 4];  // [column][row/4] dwords, swizzled
     __shared__ uint32_t red[CAST_THREADS / 64];
 
     const int t = threadIdx.x;
     const int a = t & 15;   // column group: columns 8a .. 8a+7 of the tile
     const int b = t >> 4;   // row group: rows 4b .. 4b+3 of each 64-row half
-    const int64_t r0 = (int64_t)blockIdx.y * CAST_TILE;
-    const int64_t c0 = (int64_t)blockIdx.x * CAST_TILE;
+    // Tiles are walked in bands of CAST_GROUP tile rows and, inside a band, in groups of CAST_GROUP tile
+    // columns: the blocks in flight then read 2 KB runs of each input row and write 1 KB runs of each
+    // transposed row, instead of one of the two walking through memory with a huge stride.
+    int ty, tx;
+    {
+        // consecutive workgroup ids go to the 8 XCDs round-robin; re-deal them so that one XCD (one L2)
+        // gets whole groups of neighbouring tiles and can merge their adjacent output segments
+        int64_t bid = blockIdx.x;
+        const int64_t nb = gridDim.x;
+        if (nb % 8 == 0) bid = (bid % 8) * (nb / 8) + bid / 8;
+        const int64_t band = bid / ((int64_t)CAST_GROUP * tiles_x);
+        const int64_t rem = bid - band * CAST_GROUP * tiles_x;
+        const int rows_in_band = (int)min((int64_t)CAST_GROUP, tiles_y - band * CAST_GROUP);
+        const int64_t gcol = rem / ((int64_t)rows_in_band * CAST_GROUP);
+        const int64_t r2 = rem - gcol * rows_in_band * CAST_GROUP;
+        const int cols_in_g = (int)min((int64_t)CAST_GROUP, tiles_x - gcol * CAST_GROUP);
+        ty = (int)(band * CAST_GROUP + r2 / cols_in_g);
+        tx = (int)(gcol * CAST_GROUP + r2 % cols_in_g);
+    }
+    const int64_t r0 = (int64_t)ty * CAST_TILE;
+    const int64_t c0 = (int64_t)tx * CAST_TILE;
     const int64_t col = c0 + 8 * a;
 
     Row8<DT> in[2][4];
@@ -160,9 +187,10 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
         for (int j = 0; j < 4; j++) {
             float f[8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) f[i] = scale_clamp<PROD>(elem<DT>(in[h][j], i), scale, fmax);
-            lo[j] = pack4<FMT>(f[0], f[1], f[2], f[3]);
-            hi[j] = pack4<FMT>(f[4], f[5], f[6], f[7]);
+            for (int i = 0; i < 8; i += 2)
+                scale_clamp2<PROD>(elem<DT>(in[h][j], i), elem<DT>(in[h][j], i + 1), scale, fmax, f[i], f[i + 1]);
+            lo[j] = cvt4_fp8<FMT>(f[0], f[1], f[2], f[3]);
+            hi[j] = cvt4_fp8<FMT>(f[4], f[5], f[6], f[7]);
             const int64_t row = r0 + 64 * h + 4 * b + j;
             if (out && row < rows && col < cols) {
                 uint8_t* p = out + row * cols + col;
@@ -220,7 +248,7 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
             uint32_t v = lane < CAST_THREADS / 64 ? red[lane] : 0u;
             m = wave_max_u32(v);
         }
-        publish_amax_cast(m, ws, amax_out, DT);
+        publish_amax_cast(m, amax_out, DT);
     }
 }
 
@@ -230,18 +258,18 @@ __global__ void cast_zero_amax_kernel(float* amax_out) {
 
 template <int DT, int PROD, int FMT>
 static int launch_cast2(bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
-                        const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, uint32_t* ws) {
-    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
-    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+                        const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, int64_t tiles_x, int64_t tiles_y) {
+    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
     return check_hip(hipGetLastError(), "cast kernel launch");
 }
 
 template <int DT, int PROD>
 static int launch_cast1(int fmt, bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols,
                         int64_t ld, const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev,
-                        uint32_t* ws) {
-    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
-    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+                        int64_t tiles_x, int64_t tiles_y) {
+    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
 }
 
 }  // namespace f8mi
@@ -257,7 +285,6 @@ extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, 
     if (product_dtype != in_dtype && product_dtype != F8MI_FP32) { set_error("f8mi_cast: product_dtype must be the input dtype or fp32"); return F8MI_ERR_INVALID_ARG; }
     if (!scale_dev) { set_error("f8mi_cast: null scale"); return F8MI_ERR_INVALID_ARG; }
     if (!out && !out_t && !amax_dev) { set_error("f8mi_cast: no output requested"); return F8MI_ERR_INVALID_ARG; }
-    if (amax_dev && !workspace) { set_error("f8mi_cast: fused amax needs a workspace"); return F8MI_ERR_INVALID_ARG; }
     if (rows == 0 || cols == 0) {
         if (amax_dev) {
             hipLaunchKernelGGL(cast_zero_amax_kernel, dim3(1), dim3(64), 0, stream, amax_dev);
@@ -267,20 +294,26 @@ extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, 
     }
     if (!x) { set_error("f8mi_cast: null tensor"); return F8MI_ERR_INVALID_ARG; }
     const int64_t ty = (rows + CAST_TILE - 1) / CAST_TILE, tx = (cols + CAST_TILE - 1) / CAST_TILE;
-    if (ty > 65535) { set_error("f8mi_cast: more than 65535*128 rows"); return F8MI_ERR_UNSUPPORTED; }
-    dim3 g((unsigned)tx, (unsigned)ty);
+    if (tx * ty > 0x7fffffffLL) { set_error("f8mi_cast: more than 2^31 tiles"); return F8MI_ERR_UNSUPPORTED; }
+    dim3 g((unsigned)(tx * ty));
+    const int64_t tiles_x = tx, tiles_y = ty;
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
     const bool vec = ((uintptr_t)x % 16 == 0) && ((ld * esz) % 16 == 0);
+    if (amax_dev) {
+        hipLaunchKernelGGL(cast_zero_amax_kernel, dim3(1), dim3(64), 0, stream, amax_dev);
+        int rc = check_hip(hipGetLastError(), "cast_zero_amax_kernel");
+        if (rc) return rc;
+    }
     const double n = (double)rows * (double)cols;
     ProfScope prof(F8MI_K_CAST, n * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
-    uint32_t* ws = (uint32_t*)workspace;
+    (void)workspace;
     if (in_dtype == F8MI_BF16) {
-        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
-        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
     }
     if (in_dtype == F8MI_FP16) {
-        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
-        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
     }
-    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, ws);
+    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
 }

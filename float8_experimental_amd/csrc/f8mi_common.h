@@ -45,6 +45,14 @@ __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
 
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_float(float_to_bf16_bits(f)); }
 
+// Two fp32 -> two bf16 (round to nearest even, NaN stays NaN) packed in one dword: one
+// v_cvt_pk_bf16_f32 instead of ~5 integer operations per value.
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f2){a, b}, bf2));
+}
+
 __device__ __forceinline__ float fp16_bits_to_float(uint32_t h) {
     return __half2float(__ushort_as_half((unsigned short)h));
 }
@@ -105,6 +113,23 @@ __device__ __forceinline__ uint32_t cvt2_fp8(float a, float b) {
         r |= (a != a ? 0x0001u : 0u) | (b != b ? 0x0100u : 0u);
     }
     return r & 0xffffu;
+}
+
+// Four fp32 -> four fp8 bytes in one dword: the second conversion writes the upper half of the
+// register the first one produced (no shift / or).
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
+    if constexpr (FMT == F8MI_E4M3FN) {
+        int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+        return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+    } else {
+        int r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+        uint32_t w = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
+        // the e5m2 instruction answers NaN with the quiet code 0x7E; torch's is 0x7F
+        const bool any_nan = (a != a) | (b != b) | (c != c) | (d != d);
+        if (any_nan) w |= (a != a ? 0x1u : 0u) | (b != b ? 0x100u : 0u) | (c != c ? 0x10000u : 0u) | (d != d ? 0x1000000u : 0u);
+        return w;
+    }
 }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

@@ -246,7 +246,7 @@ class Float8Linear(torch.nn.Linear):
     def _autocast_input(self, input: torch.Tensor) -> torch.Tensor:
         # what F.linear's autocast rule would do to the activation (reference :245-249)
         if torch.is_autocast_enabled():
-            input = input.to(torch.get_autocast_gpu_dtype())
+            input = input.to(torch.get_autocast_dtype('cuda'))
         return input
 
     def float8_pre_forward(self, input):

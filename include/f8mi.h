@@ -94,7 +94,8 @@ int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_t ld, int i
  *   out_t          cols x rows bytes, dense (the transpose); may be NULL
  *   amax_dev       if not NULL, max|x| of THIS call is stored there (fused
  *                  amax for hp_tensor_to_float8_delayed,
- *                  float8_scaling_utils.py:65-96); needs `workspace`
+ *                  float8_scaling_utils.py:65-96)
+ *   workspace      reserved; may be NULL
  */
 int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
               int product_dtype, int fp8_fmt, uint8_t* out, uint8_t* out_t, float* amax_dev, void* workspace,
