@@ -1,0 +1,152 @@
+// Pieces shared by the two fp8 GEMM kernels (register-staged and LDS-DMA): tile constants,
+// fragment reads, output conversion and the C epilogue.
+#pragma once
+#include <type_traits>
+
+#include "f8mi_common.h"
+
+namespace f8mi {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int GEMM_THREADS = 256;
+constexpr int STAGE_BYTES = (BM + BN) * BK;  // 64 KB
+constexpr int EPI_PITCH = 128 * 2 + 16;      // bytes per row of a wave's 128 x 128 2-byte output tile in LDS
+constexpr int EPI_BYTES = 4 * 128 * EPI_PITCH;
+constexpr int GEMM_LDS = 2 * STAGE_BYTES > EPI_BYTES ? 2 * STAGE_BYTES : EPI_BYTES;
+constexpr int GROUP_M = 8;
+constexpr int NUM_XCD = 8;
+
+#define F8MI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Workgroup barrier that waits for this wave's LDS traffic only.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+__device__ __forceinline__ v8i read_frag(const uint8_t* p0, const uint8_t* p1) {
+    const uint4 lo = *(const uint4*)p0;
+    const uint4 hi = *(const uint4*)p1;
+    return (v8i){(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+}
+
+template <int C_DT>
+__device__ __forceinline__ float load_bias(const void* bias, int col) {
+    if constexpr (C_DT == F8MI_BF16) return bf16_bits_to_float(((const uint16_t*)bias)[col]);
+    else if constexpr (C_DT == F8MI_FP16) return fp16_bits_to_float(((const uint16_t*)bias)[col]);
+    else return ((const float*)bias)[col];
+}
+
+// two fp32 -> two packed 2-byte outputs (round to nearest even)
+template <int C_DT>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    if constexpr (C_DT == F8MI_BF16) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        bf2 r = __builtin_convertvector((f2){a, b}, bf2);
+        return __builtin_bit_cast(uint32_t, r);
+    } else {
+        return (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+    }
+}
+
+// Scales a workgroup's 256 x 256 accumulators by 1 / (sa * sb), adds the bias, converts and writes C.
+// acc[tj][ti] is the 32 x 32 tile (row block ti, column block tj) of this wave's 128 x 128 quarter
+// as left by MFMA(first = Bt rows, second = A rows): lane holds row lane%32 and columns
+// 8*(e/4) + 4*(lane/32) + e%4.  2-byte outputs go through a padded LDS tile per wave so that C is
+// written with 16-byte stores; `smem` must be free for that (EPI_BYTES) when every wave arrives.
+template <int C_DT>
+__device__ __forceinline__ void store_c_tile(v16f (&acc)[4][4], uint8_t* smem, int m0, int n0, int M, int N,
+                                             const float* __restrict__ sa_dev, const float* __restrict__ sb_dev,
+                                             void* __restrict__ C, int64_t ldc, const void* __restrict__ bias,
+                                             int c_vec_ok) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
+    const int lm = lane & 31, lh = lane >> 5;
+    const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
+
+    if constexpr (C_DT == F8MI_FP32) {
+        // 4 consecutive columns per lane = one 16-byte store
+        float* Cf = (float*)C;
+#pragma unroll
+        for (int ti = 0; ti < 4; ti++) {
+            const int row = wrow0 + ti * 32 + lm;
+#pragma unroll
+            for (int tj = 0; tj < 4; tj++) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int col = wcol0 + tj * 32 + 8 * g + 4 * lh;
+                    if (row >= M || col >= N) continue;
+                    float v[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        v[r] = acc[tj][ti][4 * g + r] * inv;
+                        if (bias && col + r < N) v[r] += load_bias<C_DT>(bias, col + r);
+                    }
+                    float* dst = Cf + (int64_t)row * ldc + col;
+                    if (c_vec_ok && col + 4 <= N) {
+                        *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (col + r < N) dst[r] = v[r];
+                    }
+                }
+            }
+        }
+    } else {
+        // all waves are done with the operand stages before they become the output staging area
+        lds_barrier();
+        uint8_t* ep = smem + wave * (128 * EPI_PITCH);
+#pragma unroll
+        for (int tj = 0; tj < 4; tj++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int cl = tj * 32 + 8 * g + 4 * lh;  // column inside the wave's 128
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (bias) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (wcol0 + cl + r < N) bv[r] = load_bias<C_DT>(bias, wcol0 + cl + r);
+                }
+#pragma unroll
+                for (int ti = 0; ti < 4; ti++) {
+                    const float v0 = acc[tj][ti][4 * g + 0] * inv + bv[0];
+                    const float v1 = acc[tj][ti][4 * g + 1] * inv + bv[1];
+                    const float v2 = acc[tj][ti][4 * g + 2] * inv + bv[2];
+                    const float v3 = acc[tj][ti][4 * g + 3] * inv + bv[3];
+                    *(uint2*)(ep + (ti * 32 + lm) * EPI_PITCH + cl * 2) = make_uint2(pack2<C_DT>(v0, v1), pack2<C_DT>(v2, v3));
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own wave's tile only: no workgroup barrier needed
+        uint16_t* Ch = (uint16_t*)C;
+        const int chunk = lane & 15, rsub = lane >> 4;
+        const int col = wcol0 + chunk * 8;
+#pragma unroll 4
+        for (int it = 0; it < 32; it++) {
+            const int rl = it * 4 + rsub;
+            const int row = wrow0 + rl;
+            const uint4 v = *(const uint4*)(ep + rl * EPI_PITCH + chunk * 16);
+            if (row < M && col < N) {
+                uint16_t* dst = Ch + (int64_t)row * ldc + col;
+                if (c_vec_ok && col + 8 <= N) {
+                    *(uint4*)dst = v;
+                } else {
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++)
+                        if (col + i < N) dst[i] = (uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+                }
+            }
+        }
+    }
+}
+
+// LDS-DMA kernel (f8mi_gemm_dma.hip).  Needs 16-byte aligned operands and row strides and K % 64 == 0, K >= 384.
+int launch_gemm_dma(int a_fmt, int b_fmt, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda,
+                    const uint8_t* Bt, int64_t ldb, int M, int N, int K, const float* sa, const float* sb, void* C,
+                    int64_t ldc, const void* bias, int tiles_m, int tiles_n, int c_vec_ok);
+
+}  // namespace f8mi

@@ -266,6 +266,34 @@ def test_gemm_shapes(nat, m, n, k):
     _gemm_check(nat, m, n, k, "e4m3", "e4m3", torch.bfloat16, seed=m + n + k)
 
 
+# The library has two GEMM kernels: 16-byte aligned operands with k % 64 == 0 and k >= 384 take the
+# LDS-DMA kernel (compiled separately for an odd and an even count of 64-deep units), everything
+# else the register-staged one.  k = 384 .. 704 walks the shortest pipelines of both parities,
+# ragged m / n exercise the clamped edge rows, 8192 a long steady state.
+@pytest.mark.parametrize("m,n,k", [(256, 256, 384), (256, 256, 448), (300, 200, 512), (257, 511, 576), (64, 96, 640),
+                                   (512, 256, 704), (1, 1, 384), (520, 264, 8192), (256, 512, 8256)])
+@pytest.mark.parametrize("out_dt", [torch.bfloat16, torch.float32])
+def test_gemm_dma_kernel_shapes(nat, m, n, k, out_dt):
+    _gemm_check(nat, m, n, k, "e5m2", "e4m3", out_dt, seed=m + n + k, bias=(m % 2 == 0))
+
+
+def test_gemm_kernels_agree_bitwise(nat):
+    """Same operands through the LDS-DMA kernel (aligned view) and the register-staged kernel (the same
+    values at a 1-byte offset, which forces the unaligned path): identical accumulation order, identical bits."""
+    m, n, k = 300, 520, 1024
+    a = _rand_fp8((m, k), torch.float8_e4m3fn, 31, 4.0).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e4m3fn, 32, 4.0).to(DEV)
+    s1 = torch.ones((), device=DEV)
+    fast = nat.gemm_nt(a, s1, bt, s1, torch.float32)
+    a_off = torch.empty(m * k + 1, dtype=torch.uint8, device=DEV)[1:].view(torch.float8_e4m3fn).view(m, k)
+    b_off = torch.empty(n * k + 1, dtype=torch.uint8, device=DEV)[1:].view(torch.float8_e4m3fn).view(n, k)
+    a_off.copy_(a)
+    b_off.copy_(bt)
+    assert a_off.data_ptr() % 16 != 0
+    slow = nat.gemm_nt(a_off, s1, b_off, s1, torch.float32)
+    assert torch.equal(fast, slow)
+
+
 @pytest.mark.parametrize("a_fmt,b_fmt", [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2"), ("e5m2", "e5m2")])
 @pytest.mark.parametrize("out_dt", [torch.bfloat16, torch.float16, torch.float32])
 def test_gemm_formats_and_output_dtypes(nat, a_fmt, b_fmt, out_dt):
