@@ -29,7 +29,9 @@ EXPORTS = (
     "f8mi_workspace_bytes",
     "f8mi_amax_scale",
     "f8mi_cast",
+    "f8mi_cast_layout",
     "f8mi_gemm_nt",
+    "f8mi_gemm_nt_kb",
     "f8mi_sync",
     "f8mi_delayed_init",
     "f8mi_prof_enable",
@@ -72,6 +74,10 @@ def lib() -> C.CDLL:
         L.f8mi_amax_scale.argtypes = [vp, i64, i64, i64, i32, i32, i32, i32, fp, fp, vp, vp]
         L.f8mi_cast.restype = i32
         L.f8mi_cast.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, vp, fp, vp, vp]
+        L.f8mi_cast_layout.restype = i32
+        L.f8mi_cast_layout.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, i32, vp, i32, fp, vp]
+        L.f8mi_gemm_nt_kb.restype = i32
+        L.f8mi_gemm_nt_kb.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_nt.restype = i32
         L.f8mi_gemm_nt.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_sync.restype = i32
@@ -167,34 +173,83 @@ def amax_scale(x: torch.Tensor, float8_dtype: torch.dtype, math_dtype: Optional[
     return amax, scale
 
 
+KB = 64          # depth of one block of the k-blocked operand layout
+KB_MIN_K = 384   # shortest contraction the k-blocked GEMM takes
+
+
+def kblock_ok(k: int) -> bool:
+    """True if a contraction of length k can use the k-blocked layout ([k/64][rows][64], see f8mi.h)."""
+    return k % KB == 0 and k >= KB_MIN_K
+
+
 def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, product_dtype: Optional[torch.dtype] = None,
-         want_out: bool = True, want_out_t: bool = False, amax_out: Optional[torch.Tensor] = None):
+         want_out: bool = True, want_out_t: bool = False, amax_out: Optional[torch.Tensor] = None,
+         out_kblock: bool = False, out_t_kblock: bool = False):
     """Saturated fp8 cast of a tensor viewed as [rows, cols=last dim].
 
     Returns (out, out_t): ``out`` has x's shape; ``out_t`` is the dense [cols, rows]
     transpose of the flattened 2-D view.  ``amax_out`` (fp32, 1 element), if given,
-    receives max|x| computed in the same pass.  See f8mi_cast.
+    receives max|x| computed in the same pass.  With ``out_kblock`` / ``out_t_kblock``
+    the respective output is k-blocked instead: shape [cols/64, rows, 64] for ``out``
+    (``out[b, r, j] == rowmajor[r, 64*b + j]``), [rows/64, cols, 64] for ``out_t``.
+    See f8mi_cast / f8mi_cast_layout.
     """
     _require_gpu(x, "x")
     assert scale.dtype == torch.float32 and scale.numel() == 1 and scale.device == x.device, "scale: 1 fp32 element on x's device"
     xs, rows, cols, ld = _as_2d(x)
     if product_dtype is None:
         product_dtype = x.dtype
-    out = torch.empty(x.shape, dtype=float8_dtype, device=x.device) if want_out else None
-    out_t = torch.empty((cols, rows), dtype=float8_dtype, device=x.device) if want_out_t else None
-    ws = None
+    out = out_t = None
+    if want_out:
+        if out_kblock:
+            assert cols % KB == 0, f"k-blocked out needs cols % {KB} == 0, got {cols}"
+            out = torch.empty((cols // KB, rows, KB), dtype=float8_dtype, device=x.device)
+        else:
+            out = torch.empty(x.shape, dtype=float8_dtype, device=x.device)
+    if want_out_t:
+        if out_t_kblock:
+            assert rows % KB == 0, f"k-blocked out_t needs rows % {KB} == 0, got {rows}"
+            out_t = torch.empty((rows // KB, cols, KB), dtype=float8_dtype, device=x.device)
+        else:
+            out_t = torch.empty((cols, rows), dtype=float8_dtype, device=x.device)
     if amax_out is not None:
         assert amax_out.dtype == torch.float32 and amax_out.numel() == 1 and amax_out.device == x.device
-        ws = workspace(x.device)
-    else:
-        _check_device(x.device)
-    rc = lib().f8mi_cast(xs.data_ptr(), rows, cols, ld, _DT[x.dtype], scale.data_ptr(), _DT[product_dtype],
-                         _F8[float8_dtype], out.data_ptr() if out is not None else None,
-                         out_t.data_ptr() if out_t is not None else None,
-                         amax_out.data_ptr() if amax_out is not None else None,
-                         ws.data_ptr() if ws is not None else None, _stream(x))
-    _check(rc, "f8mi_cast")
+    _check_device(x.device)
+    rc = lib().f8mi_cast_layout(xs.data_ptr(), rows, cols, ld, _DT[x.dtype], scale.data_ptr(), _DT[product_dtype],
+                                _F8[float8_dtype], out.data_ptr() if out is not None else None, int(out_kblock),
+                                out_t.data_ptr() if out_t is not None else None, int(out_t_kblock),
+                                amax_out.data_ptr() if amax_out is not None else None, _stream(x))
+    _check(rc, "f8mi_cast_layout")
     return out, out_t
+
+
+def gemm_nt_kb(a_kb: torch.Tensor, a_scale: torch.Tensor, bt_kb: torch.Tensor, b_scale: torch.Tensor,
+               out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gemm_nt on k-blocked operands: ``a_kb`` fp8 [k/64, m, 64], ``bt_kb`` fp8 [k/64, n, 64], both contiguous.
+
+    Same result bits as gemm_nt on the row-major operands.  See f8mi_gemm_nt_kb.
+    """
+    _require_gpu(a_kb, "a_kb")
+    _require_gpu(bt_kb, "bt_kb")
+    assert a_kb.dim() == 3 and bt_kb.dim() == 3 and a_kb.shape[2] == KB and bt_kb.shape[2] == KB and a_kb.shape[0] == bt_kb.shape[0], \
+        f"k-blocked operands are [k/64, rows, 64], got {tuple(a_kb.shape)} and {tuple(bt_kb.shape)}"
+    assert a_kb.is_contiguous() and bt_kb.is_contiguous(), "k-blocked operands must be contiguous"
+    assert a_kb.dtype in _F8 and bt_kb.dtype in _F8, "operands must be float8_e4m3fn / float8_e5m2"
+    m, n, k = a_kb.shape[1], bt_kb.shape[1], a_kb.shape[0] * KB
+    for s in (a_scale, b_scale):
+        assert s.dtype == torch.float32 and s.numel() == 1 and s.device == a_kb.device, "scales: 1 fp32 element on the operands' device"
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a_kb.device)
+    else:
+        assert out.shape == (m, n) and out.dtype == out_dtype and out.is_contiguous()
+    if bias is not None:
+        assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a_kb.device
+    _check_device(a_kb.device)
+    rc = lib().f8mi_gemm_nt_kb(a_kb.data_ptr(), _F8[a_kb.dtype], bt_kb.data_ptr(), _F8[bt_kb.dtype], m, n, k,
+                               a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
+                               bias.data_ptr() if bias is not None else None, _stream(a_kb))
+    _check(rc, "f8mi_gemm_nt_kb")
+    return out
 
 
 def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: torch.Tensor, out_dtype: torch.dtype,

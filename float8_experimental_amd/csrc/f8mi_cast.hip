@@ -132,7 +132,8 @@ template <int DT, int PROD, int FMT, bool VEC>
 __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
                                                             int64_t ld, const float* __restrict__ scale_dev,
                                                             uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
-                                                            float* amax_out, int64_t tiles_x, int64_t tiles_y) {
+                                                            float* amax_out, int64_t tiles_x, int64_t tiles_y,
+                                                            int out_kb, int out_t_kb) {
     __shared__ uint32_t tileT[CAST_TILE * CAST_TILE / 4];  // [column][row/4] dwords, swizzled
     __shared__ uint32_t red[CAST_THREADS / 64];
 
@@ -193,7 +194,8 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
             hi[j] = cvt4_fp8<FMT>(f[4], f[5], f[6], f[7]);
             const int64_t row = r0 + 64 * h + 4 * b + j;
             if (out && row < rows && col < cols) {
-                uint8_t* p = out + row * cols + col;
+                // k-blocked: [cols/64][rows][64] (cols % 64 == 0, checked by the host)
+                uint8_t* p = out_kb ? out + ((col >> 6) * rows + row) * 64 + (col & 63) : out + row * cols + col;
                 if (out_vec) {  // cols % 8 == 0 implies col + 8 <= cols
                     *(uint2*)p = make_uint2(lo[j], hi[j]);
                 } else {
@@ -226,7 +228,8 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
             const int64_t gc = c0 + c;
             const int64_t gr = r0 + 16 * q;
             if (gc < cols && gr < rows) {
-                uint8_t* dst = out_t + gc * rows + gr;
+                // k-blocked: [rows/64][cols][64] (rows % 64 == 0, checked by the host)
+                uint8_t* dst = out_t_kb ? out_t + ((gr >> 6) * cols + gc) * 64 + (gr & 63) : out_t + gc * rows + gr;
                 if (t_vec) {  // rows % 16 == 0 implies gr + 16 <= rows
                     *(uint4*)dst = v;
                 } else {
@@ -258,28 +261,32 @@ __global__ void cast_zero_amax_kernel(float* amax_out) {
 
 template <int DT, int PROD, int FMT>
 static int launch_cast2(bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
-                        const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, int64_t tiles_x, int64_t tiles_y) {
-    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
-    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+                        const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb) {
+    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
     return check_hip(hipGetLastError(), "cast kernel launch");
 }
 
 template <int DT, int PROD>
 static int launch_cast1(int fmt, bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols,
                         int64_t ld, const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev,
-                        int64_t tiles_x, int64_t tiles_y) {
-    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
-    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+                        int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb) {
+    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
 }
 
 }  // namespace f8mi
 
 using namespace f8mi;
 
-extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
-                         int product_dtype, int fp8_fmt, uint8_t* out, uint8_t* out_t, float* amax_dev,
-                         void* workspace, void* stream_) {
+extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype,
+                                const float* scale_dev, int product_dtype, int fp8_fmt, uint8_t* out, int out_layout,
+                                uint8_t* out_t, int out_t_layout, float* amax_dev, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
+    if ((out_layout != F8MI_LAYOUT_ROWMAJOR && out_layout != F8MI_LAYOUT_KBLOCK64) || (out_t_layout != F8MI_LAYOUT_ROWMAJOR && out_t_layout != F8MI_LAYOUT_KBLOCK64)) { set_error("f8mi_cast: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
+    if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
+    if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
+    const int out_kb = out_layout == F8MI_LAYOUT_KBLOCK64, out_t_kb = out_t_layout == F8MI_LAYOUT_KBLOCK64;
     if (rows < 0 || cols < 0 || ld < cols) { set_error("f8mi_cast: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
     if (in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
     if (product_dtype != in_dtype && product_dtype != F8MI_FP32) { set_error("f8mi_cast: product_dtype must be the input dtype or fp32"); return F8MI_ERR_INVALID_ARG; }
@@ -306,14 +313,21 @@ extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, 
     }
     const double n = (double)rows * (double)cols;
     ProfScope prof(F8MI_K_CAST, n * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
-    (void)workspace;
     if (in_dtype == F8MI_BF16) {
-        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
-        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
     }
     if (in_dtype == F8MI_FP16) {
-        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
-        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
     }
-    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y);
+    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+}
+
+extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
+                         int product_dtype, int fp8_fmt, uint8_t* out, uint8_t* out_t, float* amax_dev,
+                         void* workspace, void* stream) {
+    (void)workspace;
+    return f8mi_cast_layout(x, rows, cols, ld, in_dtype, scale_dev, product_dtype, fp8_fmt, out, F8MI_LAYOUT_ROWMAJOR, out_t,
+                            F8MI_LAYOUT_ROWMAJOR, amax_dev, stream);
 }

@@ -305,9 +305,30 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     // F8MI_GEMM_IMPL=staged forces the register-staged kernel (for comparison runs)
     static const bool force_staged = [] { const char* e = getenv("F8MI_GEMM_IMPL"); return e && !strcmp(e, "staged"); }();
     if (aligned && K >= 384 && K % 64 == 0 && !force_staged)
-        return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+        return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_gemm1<0, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_gemm1<1, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_gemm1<0, 1>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     return launch_gemm1<1, 1>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+}
+
+extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t m, int64_t n, int64_t k,
+                               const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
+                               const void* bias_dev, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (m < 0 || n < 0 || k < 0 || ldc < n) { set_error("f8mi_gemm_nt_kb: bad shape m=%lld n=%lld k=%lld ldc=%lld", (long long)m, (long long)n, (long long)k, (long long)ldc); return F8MI_ERR_INVALID_ARG; }
+    if (a_fmt < 0 || a_fmt > 1 || b_fmt < 0 || b_fmt > 1 || c_dtype < 0 || c_dtype > 2) { set_error("f8mi_gemm_nt_kb: unknown format/dtype code"); return F8MI_ERR_INVALID_ARG; }
+    if (k % 64 != 0 || k < 384) { set_error("f8mi_gemm_nt_kb: k-blocked operands need k %% 64 == 0 and k >= 384 (k=%lld)", (long long)k); return F8MI_ERR_UNSUPPORTED; }
+    if (m == 0 || n == 0) return F8MI_OK;
+    if (!a || !bt || !c || !scale_a_dev || !scale_b_dev) { set_error("f8mi_gemm_nt_kb: null pointer"); return F8MI_ERR_INVALID_ARG; }
+    if ((uintptr_t)a % 16 != 0 || (uintptr_t)bt % 16 != 0) { set_error("f8mi_gemm_nt_kb: operands must be 16-byte aligned"); return F8MI_ERR_UNSUPPORTED; }
+    if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff - BK) { set_error("f8mi_gemm_nt_kb: dimension over 2^31"); return F8MI_ERR_UNSUPPORTED; }
+    const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    if (tiles_m * tiles_n > 0x7fffffff) { set_error("f8mi_gemm_nt_kb: too many tiles"); return F8MI_ERR_UNSUPPORTED; }
+    const int64_t csz = c_dtype == F8MI_FP32 ? 4 : 2;
+    const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
+    dim3 g((unsigned)(tiles_m * tiles_n));
+    ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
+    return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
+                           (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
 }

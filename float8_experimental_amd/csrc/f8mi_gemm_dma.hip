@@ -47,10 +47,12 @@ __device__ __forceinline__ void wait_dma() {
 
 template <int AF, int BF, int C_DT, bool ODD>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma_kernel(
-    const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ Bt, int64_t ldb, int M, int N, int K,
-    const float* __restrict__ sa_dev, const float* __restrict__ sb_dev, void* __restrict__ C, int64_t ldc,
-    const void* __restrict__ bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    const uint8_t* __restrict__ A, int64_t lda, int64_t a_unit, const uint8_t* __restrict__ Bt, int64_t ldb, int64_t b_unit,
+    int M, int N, int K, const float* __restrict__ sa_dev, const float* __restrict__ sb_dev, void* __restrict__ C,
+    int64_t ldc, const void* __restrict__ bias, int tiles_m, int tiles_n, int c_vec_ok) {
     extern __shared__ __align__(16) uint8_t smem[];
+    // lda / ldb: bytes from one operand row to the next; a_unit / b_unit: bytes from one 64-deep unit
+    // to the next.  Row-major operands: (row stride, 64); k-blocked [K/64][rows][64]: (64, rows*64).
 
     // ---- which tile (same walk as the register-staged kernel)
     int lid = blockIdx.x;
@@ -79,22 +81,22 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma_kernel(
         a_voff[i] = (uint32_t)(min(r, M - 1 - m0) * lda) + dpiece * 16;  // rows past the edge re-read the last row
         b_voff[i] = (uint32_t)(min(r, N - 1 - n0) * ldb) + dpiece * 16;
     }
-    const uint8_t* a_ptr = A + (int64_t)m0 * lda;  // advanced by UK per issued unit
+    const uint8_t* a_ptr = A + (int64_t)m0 * lda;  // advanced by one unit per issued unit
     const uint8_t* b_ptr = Bt + (int64_t)n0 * ldb;
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t dma_lds = lds0 + wave * 4096;  // + slot*SLOT_BYTES + (Bt ? BM*UK : 0) + i*1024
-    // A unit's 8 DMAs are issued as 4 pairs (A rows, A rows, Bt rows, Bt rows), each pair between
-    // two MFMAs: a burst would hold the wave (and its MFMAs) until the load unit has taken them all.
+    // A unit's 8 DMAs (d = 0..3: A rows, 4..7: Bt rows) are issued one at a time between MFMAs, two per
+    // MFMA group, waves 0,1 after the group's 1st and 3rd MFMA and waves 2,3 after its 2nd and 4th: a
+    // burst would hold the wave (and its MFMAs) until the load unit, which the four waves share, has
+    // taken them all.
     uint32_t refill_dst = 0;  // LDS address of this wave's part of the slot being refilled
-    auto issue_pair = [&](int q) __attribute__((always_inline)) {
-        if (q == 0) { dma16(a_ptr, a_voff[0], refill_dst); dma16(a_ptr, a_voff[1], refill_dst + 1024); }
-        if (q == 1) { dma16(a_ptr, a_voff[2], refill_dst + 2048); dma16(a_ptr, a_voff[3], refill_dst + 3072); }
-        if (q == 2) { dma16(b_ptr, b_voff[0], refill_dst + BM * UK); dma16(b_ptr, b_voff[1], refill_dst + BM * UK + 1024); }
-        if (q == 3) {
-            dma16(b_ptr, b_voff[2], refill_dst + BM * UK + 2048);
-            dma16(b_ptr, b_voff[3], refill_dst + BM * UK + 3072);
-            a_ptr += UK;
-            b_ptr += UK;
+    const bool late = wave >= 2;
+    auto issue_one = [&](int d) __attribute__((always_inline)) {
+        if (d < 4) dma16(a_ptr, a_voff[d], refill_dst + d * 1024);
+        else dma16(b_ptr, b_voff[d - 4], refill_dst + BM * UK + (d - 4) * 1024);
+        if (d == 7) {
+            a_ptr += a_unit;
+            b_ptr += b_unit;
         }
     };
 
@@ -130,9 +132,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma_kernel(
 #pragma unroll
     for (int x = 0; x < NSLOT; x++) {
         refill_dst = dma_lds + x * SLOT_BYTES;
-        issue_pair(0);
-        issue_pair(1);
-        if (x < NSLOT - 1) { issue_pair(2); issue_pair(3); }
+#pragma unroll
+        for (int d = 0; d < (x < NSLOT - 1 ? 8 : 4); d++) issue_one(d);
     }
     asm volatile("s_waitcnt vmcnt(28)" ::: "memory");
     lds_barrier();
@@ -165,13 +166,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma_kernel(
             }
             if (g == 3 && HAS_NEXT) { fb[P ^ 1][3] = frag_b(nxt, 3); fa[0] = frag_a(nxt, 0); }
             const bool dma_here = g < 2 ? PENDING : REFILL;
-            const int q = g < 2 ? 2 + g : g - 2;  // groups 0,1: Bt pairs of the refill in progress; 2,3: A pairs of the new one
+            const int d0 = g < 2 ? 4 + 2 * g : 2 * (g - 2);  // groups 0,1 finish the refill in progress, 2,3 start the new one
 #pragma unroll
             for (int tj = 0; tj < 4; tj++) {
                 acc[tj][g] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[P][tj], fa[g], acc[tj][g], BF, AF, 0, 0, 0, 0);
                 F8MI_SCHED_FENCE();
-                if (tj == 1 && dma_here) {
-                    issue_pair(q);
+                if (dma_here) {
+                    if (late == (bool)(tj & 1)) issue_one(d0 + (tj >> 1));
                     F8MI_SCHED_FENCE();
                 }
             }
@@ -209,8 +210,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma_kernel(
 }
 
 template <int AF, int BF, int C_DT, bool ODD>
-static int launch_dma4(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, const uint8_t* Bt, int64_t ldb, int M,
-                       int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
+static int launch_dma4(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb,
+                       int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
                        int tiles_m, int tiles_n, int c_vec_ok) {
     static bool attr_done = false;
     auto kern = gemm_nt_dma_kernel<AF, BF, C_DT, ODD>;
@@ -219,35 +220,35 @@ static int launch_dma4(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda
         if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, g, dim3(GEMM_THREADS), DMA_LDS, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias,
+    hipLaunchKernelGGL(kern, g, dim3(GEMM_THREADS), DMA_LDS, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias,
                        tiles_m, tiles_n, c_vec_ok);
     return check_hip(hipGetLastError(), "gemm (LDS-DMA) kernel launch");
 }
 
 template <int AF, int BF, int C_DT>
-static int launch_dma3(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, const uint8_t* Bt, int64_t ldb, int M,
-                       int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
+static int launch_dma3(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb,
+                       int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
                        int tiles_m, int tiles_n, int c_vec_ok) {
-    if ((K / UK - NSLOT) & 1) return launch_dma4<AF, BF, C_DT, true>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
-    return launch_dma4<AF, BF, C_DT, false>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if ((K / UK - NSLOT) & 1) return launch_dma4<AF, BF, C_DT, true>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch_dma4<AF, BF, C_DT, false>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
 }
 
 template <int AF, int BF>
-static int launch_dma2(int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, const uint8_t* Bt,
-                       int64_t ldb, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
+static int launch_dma2(int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt,
+                       int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
                        const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
-    if (c_dtype == F8MI_BF16) return launch_dma3<AF, BF, F8MI_BF16>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
-    if (c_dtype == F8MI_FP16) return launch_dma3<AF, BF, F8MI_FP16>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
-    return launch_dma3<AF, BF, F8MI_FP32>(g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (c_dtype == F8MI_BF16) return launch_dma3<AF, BF, F8MI_BF16>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (c_dtype == F8MI_FP16) return launch_dma3<AF, BF, F8MI_FP16>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch_dma3<AF, BF, F8MI_FP32>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
 }
 
-int launch_gemm_dma(int a_fmt, int b_fmt, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda,
-                    const uint8_t* Bt, int64_t ldb, int M, int N, int K, const float* sa, const float* sb, void* C,
+int launch_gemm_dma(int a_fmt, int b_fmt, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
+                    const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                     int64_t ldc, const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
-    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_dma2<0, 0>(c_dtype, g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
-    if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_dma2<1, 0>(c_dtype, g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
-    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_dma2<0, 1>(c_dtype, g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
-    return launch_dma2<1, 1>(c_dtype, g, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_dma2<0, 0>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_dma2<1, 0>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_dma2<0, 1>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch_dma2<1, 1>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
 }
 
 }  // namespace f8mi

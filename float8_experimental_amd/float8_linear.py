@@ -62,69 +62,87 @@ class _DelayedBuffers:
 
 
 def _cast_for_gemm(t2d: torch.Tensor, float8_dtype, delayed: Optional[_DelayedBuffers], is_initialized: bool,
-                   want_row: bool, want_t: bool):
-    """fp8 copies of a 2-D tensor for the GEMMs: (row-major, transposed, scale).
+                   want_row: bool, want_t: bool, row_kb: bool = False, t_kb: bool = False):
+    """fp8 copies of a 2-D tensor for the GEMMs: (as is, transposed, scale).
 
     dynamic: one amax+scale launch, one cast launch (float8_utils.py:115-120 +
     float8_tensor.py:158-159 of the reference); delayed: first-iteration init if needed,
     then ONE launch that casts with the existing scale and records this step's amax
-    (float8_scaling_utils.py:65-125).
+    (float8_scaling_utils.py:65-125).  ``row_kb`` / ``t_kb`` ask for the k-blocked layout
+    of the respective copy (same bytes, placed [k/64][rows][64] for the GEMM that contracts it).
     """
     if delayed is None:
         _, scale = _native.amax_scale(t2d, float8_dtype, want_amax=False)
-        row, tr = _native.cast(t2d, scale, float8_dtype, product_dtype=t2d.dtype, want_out=want_row, want_out_t=want_t)
+        row, tr = _native.cast(t2d, scale, float8_dtype, product_dtype=t2d.dtype, want_out=want_row, want_out_t=want_t,
+                               out_kblock=row_kb, out_t_kblock=t_kb)
         return row, tr, scale
     if not is_initialized:
         _native.amax_scale(t2d, float8_dtype, want_scale=False, amax_out=delayed.amax)
         _native.delayed_init(delayed.amax, delayed.history, delayed.scale, float8_dtype, t2d.dtype == torch.float16)
     row, tr = _native.cast(t2d, delayed.scale, float8_dtype, product_dtype=torch.float32, want_out=want_row,
-                           want_out_t=want_t, amax_out=delayed.amax)
+                           want_out_t=want_t, amax_out=delayed.amax, out_kblock=row_kb, out_t_kblock=t_kb)
     return row, tr, delayed.scale
 
 
+def _gemm(a8, sa, b8, sb, out_dtype, kb: bool):
+    return _native.gemm_nt_kb(a8, sa, b8, sb, out_dtype) if kb else _native.gemm_nt(a8, sa, b8, sb, out_dtype)
+
+
 class _float8_linear_fn(torch.autograd.Function):
-    """y = x W^T with every matmul of forward and backward in fp8 (no bias)."""
+    """y = x W^T with every matmul of forward and backward in fp8 (no bias).
+
+    Each of the three GEMMs contracts a different dimension (in_features, out_features,
+    tokens); where that length allows it (a multiple of 64, at least 384) both of its
+    operands are produced k-blocked by the cast kernel, which is the GEMM's fastest input.
+    """
 
     @staticmethod
     def forward(ctx, x, weight, mod, is_amax_initialized):
         k = x.shape[-1]
         x2 = x.reshape(-1, k)
+        m, n = x2.shape[0], weight.shape[0]
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         emulate = mod.linear_mm_config.output.emulate
+        emulate_bw = mod.linear_mm_config.grad_input.emulate or mod.linear_mm_config.grad_weight.emulate
+        kb_fwd = not emulate and _native.kblock_ok(k)      # y = x W^T contracts in_features
+        kb_dx = not emulate_bw and _native.kblock_ok(n)    # dx = dy W contracts out_features
+        kb_dw = not emulate_bw and _native.kblock_ok(m)    # dw = dy^T x contracts tokens
         dl = mod._delayed_buffers
-        x8, x8t, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, need_dw)
-        w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx)
+        x8, x8t, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, need_dw, kb_fwd, kb_dw)
+        w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx, kb_fwd, kb_dx)
         if emulate:
             y = mm_float8_emulated(x8, sx, w8.t(), sw, x.dtype)
         else:
-            y = _native.gemm_nt(x8, sx, w8, sw, x.dtype)
+            y = _gemm(x8, sx, w8, sw, x.dtype, kb_fwd)
         ctx.mod = mod
         ctx.is_amax_initialized = is_amax_initialized
         ctx.x_shape = x.shape
+        ctx.kb = (kb_dx, kb_dw)
         ctx.save_for_backward(x8t, w8t, sx, sw)
-        return y.reshape(*x.shape[:-1], weight.shape[0])
+        return y.reshape(*x.shape[:-1], n)
 
     @staticmethod
     def backward(ctx, dy):
         x8t, w8t, sx, sw = ctx.saved_tensors
         mod = ctx.mod
+        kb_dx, kb_dw = ctx.kb
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         dy2 = dy.reshape(-1, dy.shape[-1])
         g8, g8t, sg = _cast_for_gemm(dy2, e5m2_dtype, mod._delayed_buffers("grad_output"), ctx.is_amax_initialized,
-                                     need_dx, need_dw)
+                                     need_dx, need_dw, kb_dx, kb_dw)
         emulate = mod.linear_mm_config.grad_input.emulate
         dx = dw = None
         if need_dx:  # grad_input = dY @ W          [M,N] x [N,K]
             if emulate:
                 dx = mm_float8_emulated(g8, sg, w8t.t(), sw, dy.dtype)
             else:
-                dx = _native.gemm_nt(g8, sg, w8t, sw, dy.dtype)
+                dx = _gemm(g8, sg, w8t, sw, dy.dtype, kb_dx)
             dx = dx.reshape(ctx.x_shape)
         if need_dw:  # grad_weight = dY^T @ x       [N,M] x [M,K]
             if emulate:
                 dw = mm_float8_emulated(g8t, sg, x8t.t(), sx, dy.dtype)
             else:
-                dw = _native.gemm_nt(g8t, sg, x8t, sx, dy.dtype)
+                dw = _gemm(g8t, sg, x8t, sx, dy.dtype, kb_dw)
         return dx, dw, None, None
 
 

@@ -119,6 +119,32 @@ int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fm
                  int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
                  int64_t ldc, const void* bias_dev, void* stream);
 
+/* ---- k-blocked operands: the layout the fused Float8Linear path keeps its fp8 copies in ----
+ * A GEMM operand with R rows and contraction length kc (a multiple of 64) is stored as
+ * [kc/64][R][64]: byte (r, k) sits at ((k/64)*R + r)*64 + k%64.  The 64-deep slab of 256 rows
+ * that a workgroup consumes per step is then 16 KB of consecutive memory instead of 256 pieces
+ * of 64 bytes, which the load unit and the L2 move measurably faster (whole cache lines, even
+ * channel spread).  The reference keeps fp8 data row-major only (float8_tensor.py:250-262,
+ * float8_ops.py:150-153); these two entry points have no counterpart there and never change
+ * values, only where bytes are put.
+ */
+#define F8MI_LAYOUT_ROWMAJOR 0
+#define F8MI_LAYOUT_KBLOCK64 1
+
+/* f8mi_cast with a layout per output.  out_layout = KBLOCK64 stores `out` as [cols/64][rows][64]
+ * (needs cols % 64 == 0), out_t_layout = KBLOCK64 stores the transpose as [rows/64][cols][64]
+ * (needs rows % 64 == 0).  Everything else as f8mi_cast. */
+int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
+                     int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
+                     float* amax_dev, void* stream);
+
+/* f8mi_gemm_nt on k-blocked operands: a = [k/64][m][64], bt = [k/64][n][64], both 16-byte
+ * aligned.  Needs k % 64 == 0 and k >= 384 (F8MI_ERR_UNSUPPORTED otherwise: keep such operands
+ * row-major and call f8mi_gemm_nt).  Same arithmetic, same result bits as f8mi_gemm_nt. */
+int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t m, int64_t n, int64_t k,
+                    const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
+                    const void* bias_dev, void* stream);
+
 /* One (layer, tensor) row of the delayed-scaling bookkeeping; all device pointers. */
 typedef struct f8mi_sync_entry {
     float* amax;    /* [1]        fp8_amax_*          */

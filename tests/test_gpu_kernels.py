@@ -180,6 +180,55 @@ def test_cast_shapes_dynamic_and_delayed(nat, dt, shape):
         assert np.array_equal(fp8_bytes(only_t), want.reshape(x2.shape).T)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+@pytest.mark.parametrize("shape", [(64, 64), (128, 192), (448, 384), (320, 1024), (1000, 128), (192, 1000), (4, 96, 256)])
+def test_cast_kblocked_layout_is_a_permutation_of_the_row_major_bytes(nat, dt, shape):
+    """k-blocked outputs ([k/64][rows][64]) hold exactly the row-major result's bytes, re-placed; where a
+    dimension is not a multiple of 64 the request is refused."""
+    co, to = _oracles()
+    x = heavy(shape, TORCH_DT[dt], 5)
+    xd = x.to(DEV)
+    rows, cols = x.numel() // shape[-1], shape[-1]
+    tdt = torch.float8_e4m3fn
+    s = to.tensor_to_scale(x, tdt).to(DEV)
+    ref, ref_t = nat.cast(xd, s, tdt, want_out_t=True)
+    ref_b, ref_tb = fp8_bytes(ref).reshape(rows, cols), fp8_bytes(ref_t)
+    row_ok, t_ok = cols % 64 == 0, rows % 64 == 0
+    amax = torch.zeros(1, dtype=torch.float32, device=DEV)
+    out, out_t = nat.cast(xd, s, tdt, want_out=row_ok, want_out_t=t_ok, out_kblock=row_ok, out_t_kblock=t_ok,
+                          amax_out=amax if (row_ok or t_ok) else None) if (row_ok or t_ok) else (None, None)
+    if row_ok:
+        assert out.shape == (cols // 64, rows, 64)
+        assert np.array_equal(fp8_bytes(out), ref_b.reshape(rows, cols // 64, 64).transpose(1, 0, 2))
+        # mixed: k-blocked out with a row-major transpose
+        o2, t2 = nat.cast(xd, s, tdt, want_out_t=True, out_kblock=True)
+        assert np.array_equal(fp8_bytes(o2), fp8_bytes(out)) and np.array_equal(fp8_bytes(t2), ref_tb)
+    else:
+        with pytest.raises(AssertionError):
+            nat.cast(xd, s, tdt, out_kblock=True)
+    if t_ok:
+        assert out_t.shape == (rows // 64, cols, 64)
+        assert np.array_equal(fp8_bytes(out_t), ref_tb.reshape(cols, rows // 64, 64).transpose(1, 0, 2))
+    else:
+        with pytest.raises(AssertionError):
+            nat.cast(xd, s, tdt, want_out=False, want_out_t=True, out_t_kblock=True)
+    if row_ok or t_ok:
+        assert amax.item() == to.tensor_to_amax(x).float().item()
+
+
+def test_cast_kblocked_refused_by_the_library_when_not_a_multiple_of_64(nat):
+    x = torch.ones(100, 96, dtype=torch.bfloat16, device=DEV)
+    s = torch.ones((), device=DEV)
+    out = torch.empty(100 * 96, dtype=torch.uint8, device=DEV)
+    L = nat.lib()
+    rc = L.f8mi_cast_layout(x.data_ptr(), 100, 96, 96, 0, s.data_ptr(), 0, 0, out.data_ptr(), 1, None, 0, None, None)
+    assert rc != 0 and b"64" in L.f8mi_last_error()
+    rc = L.f8mi_cast_layout(x.data_ptr(), 100, 96, 96, 0, s.data_ptr(), 0, 0, None, 0, out.data_ptr(), 1, None, None)
+    assert rc != 0
+    rc = L.f8mi_cast_layout(x.data_ptr(), 100, 96, 96, 0, s.data_ptr(), 0, 0, out.data_ptr(), 7, None, 0, None, None)
+    assert rc != 0
+
+
 def test_cast_row_strided_and_c_oracle(nat):
     co, to = _oracles()
     base = heavy((70, 400), torch.bfloat16, 4)
@@ -292,6 +341,32 @@ def test_gemm_kernels_agree_bitwise(nat):
     assert a_off.data_ptr() % 16 != 0
     slow = nat.gemm_nt(a_off, s1, b_off, s1, torch.float32)
     assert torch.equal(fast, slow)
+
+
+def _to_kb(t):
+    """[rows, k] fp8 -> k-blocked [k/64, rows, 64] (byte permutation on the device)."""
+    rows, k = t.shape
+    return t.view(torch.uint8).view(rows, k // 64, 64).permute(1, 0, 2).contiguous().view(t.dtype)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 384), (300, 200, 448), (257, 511, 576), (1, 7, 640), (520, 264, 8192), (1024, 768, 2048)])
+def test_gemm_kblocked_equals_row_major_bitwise(nat, m, n, k):
+    a = _rand_fp8((m, k), torch.float8_e5m2, m + k, 4.0).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e4m3fn, n + k, 4.0).to(DEV)
+    sa, sb = torch.tensor(3.0, device=DEV), torch.tensor(0.5, device=DEV)
+    bias = (torch.randn(n) * 3).to(torch.bfloat16).to(DEV)
+    for out_dt, b in ((torch.bfloat16, bias), (torch.float32, None), (torch.float16, None)):
+        want = nat.gemm_nt(a, sa, bt, sb, out_dt, bias=b)
+        got = nat.gemm_nt_kb(_to_kb(a), sa, _to_kb(bt), sb, out_dt, bias=b)
+        assert torch.equal(got, want), (m, n, k, out_dt)
+
+
+def test_gemm_kblocked_refuses_short_or_ragged_k(nat):
+    s1 = torch.ones((), device=DEV)
+    for k in (64, 320):
+        a = torch.zeros(k // 64, 8, 64, dtype=torch.float8_e4m3fn, device=DEV)
+        with pytest.raises(nat.Float8NativeError):
+            nat.gemm_nt_kb(a, s1, a, s1, torch.bfloat16)
 
 
 @pytest.mark.parametrize("a_fmt,b_fmt", [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2"), ("e5m2", "e5m2")])

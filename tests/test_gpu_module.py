@@ -201,6 +201,31 @@ def test_fused_forward_equals_the_composed_reference_pipeline(f8, scaling):
                 assert torch.equal(b1, b2), n1
 
 
+@pytest.mark.parametrize("scaling", [("dyn", "dyn", "dyn"), ("del", "del", "del")])
+@pytest.mark.parametrize("m,k,n", [(512, 384, 448), (384, 512, 200), (100, 448, 384), (448, 200, 640)])
+def test_fused_path_with_k_blocked_operands_equals_the_composed_pipeline(f8, scaling, m, k, n):
+    """Sizes at which some or all of the three GEMMs take k-blocked operands (contraction a multiple
+    of 64 and >= 384) against the composed, row-major pipeline: identical bits everywhere."""
+    torch.manual_seed(2)
+    lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
+    a = f8.Float8Linear.from_float(copy.deepcopy(lin), config=_cfg(f8, *scaling)).to(DEV)
+    b = f8.Float8Linear.from_float(copy.deepcopy(lin), config=_cfg(f8, *scaling)).to(DEV)
+    for it in range(2):
+        x = (torch.randn(m, k) * (it + 1)).to(torch.bfloat16).to(DEV)
+        dy = torch.randn(m, n).to(torch.bfloat16).to(DEV)
+        outs = []
+        for mod, fwd in ((a, a.forward), (b, b.forward_composed)):
+            if "del" in scaling:
+                f8.sync_float8_amax_and_scale_history(mod)
+            xi = x.clone().requires_grad_()
+            mod.weight.grad = None
+            y = fwd(xi)
+            y.backward(dy)
+            outs.append((y, xi.grad, mod.weight.grad))
+        for u, v in zip(*outs):
+            assert torch.equal(u, v)
+
+
 # --------------------------------------------------------------- config 1
 
 
