@@ -281,6 +281,17 @@ static int launch_gemm1(bool aligned, int c_dtype, dim3 g, hipStream_t stream, c
 
 using namespace f8mi;
 
+// 0: default choice, 1: register-staged kernel only, 2: no 16x16x128 kernel
+static int gemm_impl() {
+    static const int v = [] {
+        const char* e = getenv("F8MI_GEMM_IMPL");
+        if (e && !strcmp(e, "staged")) return 1;
+        if (e && !strcmp(e, "dma32")) return 2;
+        return 0;
+    }();
+    return v;
+}
+
 extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fmt, int64_t ldb, int64_t m,
                             int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c,
                             int c_dtype, int64_t ldc, const void* bias_dev, void* stream_) {
@@ -302,10 +313,12 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     const uint8_t* A = (const uint8_t*)a;
     const uint8_t* B = (const uint8_t*)bt;
     const int M = (int)m, N = (int)n, K = (int)k;
-    // F8MI_GEMM_IMPL=staged forces the register-staged kernel (for comparison runs)
-    static const bool force_staged = [] { const char* e = getenv("F8MI_GEMM_IMPL"); return e && !strcmp(e, "staged"); }();
-    if (aligned && K >= 384 && K % 64 == 0 && !force_staged)
+    // F8MI_GEMM_IMPL=staged forces the register-staged kernel, =dma32 the 32x32x64 LDS-DMA kernel (comparison runs)
+    if (aligned && K >= 384 && K % 64 == 0 && gemm_impl() != 1) {
+        if (K % 128 == 0 && gemm_impl() != 2)
+            return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
         return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    }
     if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_gemm1<0, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_gemm1<1, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_gemm1<0, 1>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
@@ -329,6 +342,9 @@ extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_f
     const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
+    if (k % 128 == 0 && gemm_impl() != 2)
+        return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
+                                 (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
                            (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
 }

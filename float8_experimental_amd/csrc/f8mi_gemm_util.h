@@ -150,5 +150,9 @@ __device__ __forceinline__ void store_c_tile(v16f (&acc)[4][4], uint8_t* smem, i
 int launch_gemm_dma(int a_fmt, int b_fmt, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                     const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb,
                     void* C, int64_t ldc, const void* bias, int tiles_m, int tiles_n, int c_vec_ok);
+// The same on the 16x16x128 MFMA (f8mi_gemm_dma16.hip); additionally needs K % 128 == 0.
+int launch_gemm_dma16(int a_fmt, int b_fmt, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
+                      const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb,
+                      void* C, int64_t ldc, const void* bias, int tiles_m, int tiles_n, int c_vec_ok);
 
 }  // namespace f8mi
