@@ -29,6 +29,11 @@ M_TOKENS = 16384
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
+# Bytes per GEMM launch that cross the L2 boundary (fetch + write), averaged over the 12 launches of a step:
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this script, each scaled by the same counter's reading for a
+# 1 GiB device copy (x2.0 and x1.0); the summary is profiles/bench_llama70b_gemm_hbm_traffic_pmc.txt.
+# Only meaningful at the default --m.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 5.87e9
 
 
 def parse():
@@ -40,6 +45,8 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-bf16", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the oracle sample")
+    p.add_argument("--calibrate-copy", action="store_true",
+                   help="also run one plain 1 GiB device-to-device copy (for scaling hardware byte counters of a profiler run)")
     return p.parse_args()
 
 
@@ -125,6 +132,13 @@ def main():
     flop_per_shape = {name: 3 * 2.0 * m * k * n for name, k, n, *_ in layers}
     flop_step = sum(flop_per_shape.values())
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- the timed region: K steps, every kernel launch bracketed by HIP events on its stream
     for _ in range(args.warmup):
         step(layers)
@@ -186,13 +200,14 @@ def main():
             "flop_convention": "3 * 2*M*K*N per shape",
         },
         "roofline": {
-            "kernel": "f8mi gemm_nt_kernel (fp8 MFMA GEMM, all 12 launches of a step)",
+            "kernel": "f8mi gemm_nt_dma16_kernel (fp8 MFMA GEMM on k-blocked operands, all 12 launches of a step)",
             "bound": "mfma",
             "achieved": gemm_tflops,
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_tflops / PEAK_FP8_TFLOPS,
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if m == M_TOKENS else None,
+            "traffic_unit": "bytes past the L2 per launch (FETCH_SIZE + WRITE_SIZE, calibrated); algorithmic: 1.035e9",
             "launches": n_gemm,
             "avg_launch_ms": ms_gemm / max(n_gemm, 1),
             "flop_per_launch": flop_gemm / max(n_gemm, 1),
