@@ -16,8 +16,8 @@
 // Two barriers per step: Q (after 6 of 8 groups; before it a wave waits until its own DMAs
 // of step t+1 have landed, after it everybody's have) and S (step boundary; everybody is done
 // reading A of step t and Bt of step t+1, whose slabs are refilled with step t+3's and step
-// t+3's right away -- 16 DMAs per wave, issued one per two MFMAs during the first half of
-// the step, about 1.75 steps ahead of their first use).
+// t+3's -- 16 DMAs per wave, issued one per four MFMAs through the step, 1 to 1.75 steps
+// ahead of their first use).
 // Requirements checked by the host: 16-byte aligned operands and strides, K % 128 == 0,
 // K >= 384.
 #include "f8mi_gemm_util.h"
@@ -155,10 +155,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
     int lid = blockIdx.x;
     const int npid = gridDim.x;
     if (npid % NUM_XCD == 0) lid = (lid % NUM_XCD) * (npid / NUM_XCD) + lid / NUM_XCD;
-    const int width = GROUP_M * tiles_n;
+    constexpr int GROUP = 4;  // tile rows per walk group: an XCD's 32 workgroups then hold 4 x 8 neighbouring tiles
+    const int width = GROUP * tiles_n;
     const int group = lid / width;
-    const int first_m = group * GROUP_M;
-    const int gsz = min(tiles_m - first_m, GROUP_M);
+    const int first_m = group * GROUP;
+    const int gsz = min(tiles_m - first_m, GROUP);
     const int tm = first_m + (lid % width) % gsz;
     const int tn = (lid % width) / gsz;
     const int m0 = tm * BM, n0 = tn * BN;
@@ -254,8 +255,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
 #pragma unroll
         for (int ti = 0; ti < 8; ti++) {
             if (ti == 6 && MODE < 2) {
-                // this wave's DMAs of step t+1 have landed (the 16 of step t+2 may be in flight) ...
-                if (MODE == 0) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+                // this wave's DMAs of step t+1 have landed (the 12 of step t+2 issued so far may be in flight) ...
+                if (MODE == 0) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
                 else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 asm volatile("s_barrier" ::: "memory");  // ... and so have everybody's; no LDS hazard here, so no wait on LDS reads
             }
@@ -267,9 +268,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
                 if (FIRST) mfma16_first<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
                 else mfma16<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
                 F8MI_SCHED_FENCE();
-                if (MODE == 0 && ti < 4 && (tj & 1) == 0) {
-                    // 16 DMAs over the first 32 MFMAs, one after every other MFMA: A slab first, then Bt
-                    const int d = ti * 4 + (tj >> 1);
+                if (MODE == 0 && (tj & 3) == 0) {
+                    // 16 DMAs over the 64 MFMAs, one after every fourth: A slab first, then Bt.  (Packed into
+                    // the first half of the step they cost 3 % more time: the four waves share one load unit.)
+                    const int d = ti * 2 + (tj >> 2);
                     if (d < 8) issue_a(d);
                     else issue_b(d - 8);
                     F8MI_SCHED_FENCE();
