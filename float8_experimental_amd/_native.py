@@ -13,7 +13,8 @@ from typing import Optional, Tuple
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libf8mi.so")
+# F8MI_LIB names another build of the library (same ABI) to load instead of the in-tree one
+LIB_PATH = os.environ.get("F8MI_LIB") or os.path.join(_HERE, "libf8mi.so")
 
 BF16, FP16, FP32 = 0, 1, 2
 E4M3FN, E5M2 = 0, 1
