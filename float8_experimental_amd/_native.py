@@ -130,7 +130,7 @@ _workspaces = {}
 
 
 def workspace(dev: torch.device) -> torch.Tensor:
-    """Zero-filled reduction workspace, one per (device, stream); kernels re-zero it themselves."""
+    """Reduction workspace of f8mi_amax_scale (per-block partial maxima), one per (device, stream)."""
     _check_device(dev)
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
     ws = _workspaces.get(key)

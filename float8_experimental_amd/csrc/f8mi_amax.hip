@@ -3,9 +3,11 @@
 // |x| is reduced on the raw bit patterns: for IEEE formats the unsigned order
 // of sign-cleared patterns is the order of the magnitudes, and every NaN
 // pattern is larger than inf, so a NaN anywhere wins the max exactly like
-// torch.max propagates it.  Each block folds its result into one word of the
-// workspace with atomicMax; the last block to finish turns the word into
-// amax + scale and zeroes the workspace again.
+// torch.max propagates it.  Each block stores its result in its own word of the
+// workspace; a second, one-block launch on the same stream reduces those words and
+// writes amax + scale.  (One word plus a "last block" ticket, both updated with
+// atomics, cost about 80 ns per block, serialised at the end of the kernel: 40 us of
+// a 90 us kernel with 512 blocks.)
 #include "f8mi_common.h"
 
 namespace f8mi {
@@ -52,23 +54,21 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* lds) {
     return m;  // valid in wave 0
 }
 
-// Fold this block's max into the workspace; the last block publishes amax/scale.
-__device__ __forceinline__ void publish_amax(uint32_t blockmax, uint32_t* ws, float* amax_out, float* scale_out,
-                                             int in_dt, int math_dt, int fmt, int orig_is_fp16) {
+// Reduces the per-block maxima and publishes amax / scale.  One block.
+__global__ __launch_bounds__(AMAX_THREADS) void amax_finalize_kernel(const uint32_t* __restrict__ ws, int nblocks,
+                                                                      float* amax_out, float* scale_out, int in_dt,
+                                                                      int math_dt, int fmt, int orig_is_fp16) {
+    __shared__ uint32_t red[AMAX_THREADS / 64];
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < nblocks; i += AMAX_THREADS) {
+        const uint32_t v = ws[i];
+        m = m > v ? m : v;
+    }
+    m = block_max_u32(m, red);
     if (threadIdx.x == 0) {
-        // the running maximum only grows: a (possibly stale) read that is already >= this block's value
-        // makes the atomic unnecessary, which keeps thousands of blocks from queueing on one address
-        if (blockmax > __atomic_load_n(&ws[WS_AMAX_BITS], __ATOMIC_RELAXED)) atomicMax(&ws[WS_AMAX_BITS], blockmax);
-        __threadfence();
-        uint32_t ticket = atomicAdd(&ws[WS_TICKET], 1u);
-        if (ticket == gridDim.x * gridDim.y - 1) {
-            __threadfence();
-            uint32_t bits = atomicExch(&ws[WS_AMAX_BITS], 0u);
-            atomicExch(&ws[WS_TICKET], 0u);
-            float amax = abs_bits_to_float(bits, in_dt);
-            if (amax_out) *amax_out = amax;
-            if (scale_out) *scale_out = amax_to_scale_dev(amax, math_dt, fmt, orig_is_fp16);
-        }
+        const float amax = abs_bits_to_float(m, in_dt);
+        if (amax_out) *amax_out = amax;
+        if (scale_out) *scale_out = amax_to_scale_dev(amax, math_dt, fmt, orig_is_fp16);
     }
 }
 
@@ -78,8 +78,7 @@ __device__ __forceinline__ void publish_amax(uint32_t blockmax, uint32_t* ws, fl
 // grid instead costs more than half of the bandwidth.)
 template <int DT>
 __global__ __launch_bounds__(AMAX_THREADS) void amax_dense_kernel(const void* __restrict__ x, int64_t n,
-                                                                   uint32_t* ws, float* amax_out, float* scale_out,
-                                                                   int math_dt, int fmt, int orig_is_fp16) {
+                                                                   uint32_t* __restrict__ ws) {
     __shared__ uint32_t red[AMAX_THREADS / 64];
     constexpr int EPV = DT == F8MI_FP32 ? 4 : 8;
     constexpr int64_t TILE = (int64_t)AMAX_THREADS * AMAX_UNROLL;
@@ -111,15 +110,13 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_dense_kernel(const void* __
         }
     }
     m = block_max_u32(m, red);
-    publish_amax(m, ws, amax_out, scale_out, DT, math_dt, fmt, orig_is_fp16);
+    if (threadIdx.x == 0) ws[blockIdx.x] = m;
 }
 
 // Any row stride / alignment: one element per thread step.
 template <int DT>
 __global__ __launch_bounds__(AMAX_THREADS) void amax_strided_kernel(const void* __restrict__ x, int64_t rows,
-                                                                     int64_t cols, int64_t ld, uint32_t* ws,
-                                                                     float* amax_out, float* scale_out, int math_dt,
-                                                                     int fmt, int orig_is_fp16) {
+                                                                     int64_t cols, int64_t ld, uint32_t* __restrict__ ws) {
     __shared__ uint32_t red[AMAX_THREADS / 64];
     uint32_t m = 0;
     const int64_t n = rows * cols;
@@ -130,7 +127,7 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_strided_kernel(const void* 
         m = m > a ? m : a;
     }
     m = block_max_u32(m, red);
-    publish_amax(m, ws, amax_out, scale_out, DT, math_dt, fmt, orig_is_fp16);
+    if (threadIdx.x == 0) ws[blockIdx.x] = m;
 }
 
 // Empty tensor: torch.max raises; we define amax = 0 so the scale is fmax/eps.
@@ -176,25 +173,32 @@ extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
     const bool dense = (ld == cols || rows == 1) && ((uintptr_t)x % 16 == 0);
     ProfScope prof(F8MI_K_AMAX, (double)n * esz, stream);
+    int64_t blocks;
     if (dense) {
         const int64_t epv = 16 / esz;
         const int64_t nvec = n / epv;
-        int64_t blocks = (nvec + (int64_t)AMAX_THREADS * AMAX_UNROLL - 1) / ((int64_t)AMAX_THREADS * AMAX_UNROLL);
-        const int64_t cap = (int64_t)cu_count() * 2;  // few, long-lived blocks: one ticket atomic each
+        blocks = (nvec + (int64_t)AMAX_THREADS * AMAX_UNROLL - 1) / ((int64_t)AMAX_THREADS * AMAX_UNROLL);
+        int64_t cap = (int64_t)cu_count() * 2;  // few, long-lived blocks, two per CU
+        if (cap > WS_WORDS) cap = WS_WORDS;
         if (blocks > cap) blocks = cap;
         if (blocks < 1) blocks = 1;
         dim3 g((unsigned)blocks), b(AMAX_THREADS);
-        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_BF16>, g, b, 0, stream, x, n, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
-        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP16>, g, b, 0, stream, x, n, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
-        else hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP32>, g, b, 0, stream, x, n, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_BF16>, g, b, 0, stream, x, n, ws);
+        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP16>, g, b, 0, stream, x, n, ws);
+        else hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP32>, g, b, 0, stream, x, n, ws);
     } else {
-        int64_t blocks = (n + AMAX_THREADS - 1) / AMAX_THREADS;
-        const int64_t cap = (int64_t)cu_count() * 8;
+        blocks = (n + AMAX_THREADS - 1) / AMAX_THREADS;
+        int64_t cap = (int64_t)cu_count() * 8;
+        if (cap > WS_WORDS) cap = WS_WORDS;
         if (blocks > cap) blocks = cap;
         dim3 g((unsigned)blocks), b(AMAX_THREADS);
-        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_strided_kernel<F8MI_BF16>, g, b, 0, stream, x, rows, cols, ld, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
-        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP16>, g, b, 0, stream, x, rows, cols, ld, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
-        else hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP32>, g, b, 0, stream, x, rows, cols, ld, ws, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_strided_kernel<F8MI_BF16>, g, b, 0, stream, x, rows, cols, ld, ws);
+        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP16>, g, b, 0, stream, x, rows, cols, ld, ws);
+        else hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP32>, g, b, 0, stream, x, rows, cols, ld, ws);
     }
-    return check_hip(hipGetLastError(), "amax kernel launch");
+    int rc = check_hip(hipGetLastError(), "amax kernel launch");
+    if (rc) return rc;
+    hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(AMAX_THREADS), 0, stream, ws, (int)blocks, amax_dev, scale_dev, in_dtype,
+                       math_dtype, fp8_fmt, orig_is_fp16);
+    return check_hip(hipGetLastError(), "amax finalize kernel launch");
 }

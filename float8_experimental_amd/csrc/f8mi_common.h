@@ -24,10 +24,8 @@ struct ProfScope {
     ~ProfScope();
 };
 
-// workspace layout (uint32 words); every kernel leaves all words zero
-constexpr int WS_AMAX_BITS = 0;  // running max of |x| bit patterns
-constexpr int WS_TICKET = 1;     // blocks that have finished
-constexpr int WS_WORDS = 8;
+// workspace (uint32 words): one partial max of |x| bit patterns per block of the amax kernel
+constexpr int WS_WORDS = 1024;
 
 // ---------------------------------------------------------------- device side
 

@@ -58,8 +58,8 @@ const char* f8mi_last_error(void);
  * Returns F8MI_ERR_ARCH when it is not a gfx950. */
 int f8mi_device_info(int device, int* cu_count, int* lds_bytes, char* arch, int arch_len);
 
-/* Bytes of the small device workspace the reducing kernels need.  The caller
- * zero-fills it ONCE; every kernel leaves it zeroed again.  One workspace must
+/* Bytes of the small device workspace f8mi_amax_scale needs (per-block partial
+ * results; 4 KB).  Its contents between calls do not matter.  One workspace must
  * not be shared by calls that can overlap in time (use one per stream). */
 size_t f8mi_workspace_bytes(void);
 
