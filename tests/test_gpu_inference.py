@@ -1,0 +1,161 @@
+"""Float8InferenceLinear on the GPU: the reference's inference flows (test/test_inference_flows.py) plus
+bit-level checks against the oracle and against the training module."""
+import copy
+import io
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from tests.helpers import fp8_bytes
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def f8():
+    if not torch.cuda.is_available():
+        pytest.fail("these tests need a GPU (run with -m gpu on an MI355X box)")
+    import float8_experimental_amd as pkg
+    from float8_experimental_amd import _native
+
+    _native.lib()
+    return pkg
+
+
+class FeedForward(nn.Module):
+    def __init__(self, d=4096, ffn=14336, bias=False):
+        super().__init__()
+        self.w1 = nn.Linear(d, ffn, bias=bias)
+        self.w3 = nn.Linear(d, ffn, bias=bias)
+        self.w2 = nn.Linear(ffn, d, bias=bias)
+
+    def forward(self, x):
+        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+
+
+def _sqnr(f8, a, b):
+    return f8.float8_utils.compute_error(a, b).item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["dynamic", "static", "weight_only"])
+def test_mlp_flows_sqnr(f8, dtype, mode):
+    """test_inference_flows.py:62-168: SQNR > 20 dB against the high-precision MLP."""
+    from float8_experimental_amd.inference import ActivationCasting, Float8InferenceLinear, QuantConfig, quantize_to_float8
+
+    torch.manual_seed(0)
+    base = FeedForward().to(DEV, dtype=dtype)
+    q = copy.deepcopy(base)
+    cfg = {"dynamic": QuantConfig(ActivationCasting.DYNAMIC),
+           "static": QuantConfig(ActivationCasting.STATIC, static_quantization_scale=torch.tensor([1.0], device=DEV)),
+           "weight_only": QuantConfig(ActivationCasting.WEIGHT_ONLY)}[mode]
+    quantize_to_float8(q, cfg)
+    n = 0
+    for m in q.modules():
+        if isinstance(m, Float8InferenceLinear):
+            assert isinstance(m.weight, f8.Float8Tensor) and m.weight.requires_grad is False
+            n += 1
+    assert n == 3
+    x = torch.randn(4, 1024, 4096, device=DEV, dtype=dtype)
+    with torch.no_grad():
+        want, got = base(x), q(x)
+    assert got.dtype == dtype and got.shape == want.shape
+    assert _sqnr(f8, want, got) > 20
+
+
+@pytest.mark.parametrize("shape,bias", [((3, 40, 512), True), ((130, 448), False), ((7, 200), True), ((64, 4096), True)])
+@pytest.mark.parametrize("static", [False, True])
+def test_fast_path_equals_the_composed_float8tensor_route_and_the_oracle(f8, shape, bias, static):
+    """The module's own route (cast in the GEMM's layout, bias in the epilogue) against the reference's
+    composition F.linear(Float8Tensor, Float8Tensor, bias), bit for bit, and against the CPU oracle."""
+    from float8_experimental_amd.inference import (ActivationCasting, Float8InferenceLinear, QuantConfig,
+                                                   cast_to_float8_e4m3_inference)
+    from oracle import torch_oracle as to
+
+    torch.manual_seed(1)
+    k, n = shape[-1], 320
+    lin = nn.Linear(k, n, bias=bias).to(torch.bfloat16)
+    sq = torch.tensor([37.0]) if static else None
+    cfg = QuantConfig(ActivationCasting.STATIC, static_quantization_scale=sq.to(DEV)) if static else QuantConfig(ActivationCasting.DYNAMIC)
+    mod = Float8InferenceLinear.from_float(copy.deepcopy(lin).to(DEV), cfg, use_fast_accum=True)
+    x = (torch.randn(shape) * 3).to(torch.bfloat16)
+    with torch.no_grad():
+        got = mod(x.to(DEV))
+        x8 = cast_to_float8_e4m3_inference(x.to(DEV), mod.linear_mm_config, static_quantization_scale=mod.static_quantization_scale)
+        composed = F.linear(x8, mod.weight, mod.bias)
+    assert torch.equal(got, composed)
+    # oracle: weight and activation bytes exact, output within the GEMM tolerance of the emulated product
+    sw = to.tensor_to_scale(lin.weight.detach(), torch.float8_e4m3fn)
+    w8 = to.cast_to_fp8(lin.weight.detach(), sw, torch.float8_e4m3fn)
+    assert np.array_equal(fp8_bytes(mod.weight._data), fp8_bytes(w8)) and mod.weight._scale.item() == sw.item()
+    x2 = x.reshape(-1, k)
+    sx = sq if static else to.tensor_to_scale(x2, torch.float8_e4m3fn)
+    xo = to.cast_to_fp8(x2, sx, torch.float8_e4m3fn)
+    assert np.array_equal(fp8_bytes(x8._data).reshape(-1, k), fp8_bytes(xo))
+    want = to.mm_emulated(xo, sx, w8.t(), sw, torch.bfloat16).float()
+    if bias:
+        want = want + lin.bias.detach().float()
+    err = (got.float().cpu().reshape(-1, n) - want).abs().max().item() / want.abs().max().item()
+    assert err <= 1e-2, err
+
+
+def test_weight_only_dequantises_and_ignores_the_bias_like_the_reference(f8):
+    from float8_experimental_amd.inference import ActivationCasting, Float8InferenceLinear, QuantConfig
+
+    torch.manual_seed(2)
+    lin = nn.Linear(256, 128, bias=True).to(DEV, dtype=torch.bfloat16)
+    mod = Float8InferenceLinear.from_float(copy.deepcopy(lin), QuantConfig(ActivationCasting.WEIGHT_ONLY), use_fast_accum=True)
+    x = torch.randn(9, 256, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        got = mod(x)
+        want = F.linear(x, mod.weight.to_original_precision())  # inference.py:104-107: no bias on this branch
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fp8_training_then_save_load_then_inference_is_bit_identical(f8, dtype):
+    """test_inference_flows.py:190-240, at a reduced width: Float8Linear training, state dict round trip
+    through torch.save / torch.load(weights_only=True) into meta-device modules, conversion to inference
+    modules: outputs equal the training modules' eval outputs exactly."""
+    from float8_experimental_amd.inference import ActivationCasting, Float8InferenceLinear, QuantConfig, quantize_to_float8
+
+    torch.manual_seed(3)
+    d, ffn = 512, 1408
+    mlp = FeedForward(d, ffn).to(DEV, dtype=torch.float32)
+    f8.convert_to_float8_training(mlp)
+    opt = torch.optim.SGD(mlp.parameters(), lr=1e-3)
+    target = torch.randn(4, 256, d, device=DEV, dtype=dtype)
+    for _ in range(5):
+        opt.zero_grad()
+        with torch.autocast("cuda", dtype=dtype, enabled=dtype != torch.float32):
+            out = mlp(torch.randn(4, 256, d, device=DEV, dtype=dtype))
+        F.mse_loss(out.float(), target.float()).backward()
+        opt.step()
+    mlp.eval()
+    mlp = mlp.to(dtype)
+    x = torch.randn(4, 256, d, device=DEV, dtype=dtype)
+    with torch.no_grad():
+        og_out = mlp(x)
+    buf = io.BytesIO()
+    torch.save(mlp.state_dict(), buf)
+    buf.seek(0)
+    with torch.device("meta"):
+        new = FeedForward(d, ffn).to(dtype=dtype)
+        f8.convert_to_float8_training(new)
+    new.load_state_dict(torch.load(buf, weights_only=True), strict=True, assign=True)
+    quantize_to_float8(new, QuantConfig(ActivationCasting.DYNAMIC))
+    assert sum(isinstance(m, Float8InferenceLinear) for m in new.modules()) == 3
+    with torch.no_grad():
+        new_out = new(x)
+    assert torch.equal(og_out, new_out)
+    # and the quantised module's own state dict survives a weights_only round trip
+    buf = io.BytesIO()
+    torch.save(new.state_dict(), buf)
+    buf.seek(0)
+    sd = torch.load(buf, weights_only=True)
+    assert isinstance(sd["w1.weight"], f8.Float8Tensor)
+    assert torch.equal(sd["w1.weight"]._data.view(torch.uint8), new.w1.weight._data.view(torch.uint8))
