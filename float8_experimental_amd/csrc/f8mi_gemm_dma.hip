@@ -1,4 +1,5 @@
-// K3, fast path: the scaled fp8 GEMM of f8mi_gemm.hip with the operands moved
+// K3, LDS-DMA path on 32x32x64 MFMAs (takes K % 128 == 64; K % 128 == 0 goes to
+// f8mi_gemm_dma16.hip): the scaled fp8 GEMM of f8mi_gemm.hip with the operands moved
 // HBM -> LDS by the load unit itself (global_load_lds_dwordx4: every lane names 16
 // bytes of global memory, the wave's 64 pieces land in 1 KB of consecutive LDS
 // starting at M0), no staging registers and no LDS writes by the waves.
@@ -11,7 +12,7 @@
 //     16 consecutive rows of one piece cover all 64 banks, so fragment reads run
 //     at the LDS's full rate.  The swizzle is applied on the global side: lane l
 //     of DMA instruction j fetches row 16j + l/4, piece (l%4) ^ ((l/16) % 4).
-//   * per unit and wave: 8 DMA instructions (4 for A, 4 for Bt), issued in pairs
+//   * per unit and wave: 8 DMA instructions (4 for A, 4 for Bt), issued one at a time
 //     between MFMAs after the barrier that ends all reads of the slot they refill,
 //     5 units ahead of the multiply (about two full K steps of latency cover).
 //   * one barrier per unit, after the second MFMA group: before it a wave has

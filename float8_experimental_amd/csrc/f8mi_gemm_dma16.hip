@@ -15,9 +15,9 @@
 //   * the A fragments are read one 8-MFMA group ahead, all through step t.
 // Two barriers per step: Q (after 6 of 8 groups; before it a wave waits until its own DMAs
 // of step t+1 have landed, after it everybody's have) and S (step boundary; everybody is done
-// reading A of step t and Bt of step t+1, whose slabs are refilled with step t+3's and step
-// t+3's -- 16 DMAs per wave, issued one per four MFMAs through the step, 1 to 1.75 steps
-// ahead of their first use).
+// reading A of step t and Bt of step t+1; during step t+1 those two slabs are refilled with
+// step t+3's A and Bt -- 16 DMAs per wave, issued one per four MFMAs through the step, 1 to
+// 1.75 steps ahead of their first use).
 // Requirements checked by the host: 16-byte aligned operands and strides, K % 128 == 0,
 // K >= 384.
 #include "f8mi_gemm_util.h"

@@ -285,6 +285,29 @@ class Float8Linear(torch.nn.Linear):
     # ---- forward ---------------------------------------------------------------------------
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
+        if torch.compiler.is_compiling():
+            return self._forward_under_compile(input)
+        return self._forward_eager(input)
+
+    def _forward_under_compile(self, input: torch.Tensor) -> torch.Tensor:
+        """What ``torch.compile`` traces: all-dynamic scaling is one custom-op node (plus the bias add);
+        anything that keeps state on the module, or carries Float8Tensors, runs outside the graph."""
+        plain = (not self.has_any_delayed_scaling and not self.config.emulate
+                 and not isinstance(self.weight, Float8Tensor) and not isinstance(input, Float8Tensor))
+        if not plain:
+            return self._forward_outside_graph(input)
+        from ._custom_ops import linear_dynamic
+
+        output = linear_dynamic(self._autocast_input(input), self.weight)
+        if self.bias is not None:
+            output = output + self.bias.to(output.dtype)
+        return output
+
+    @torch._dynamo.disable
+    def _forward_outside_graph(self, input: torch.Tensor) -> torch.Tensor:
+        return self._forward_eager(input)
+
+    def _forward_eager(self, input: torch.Tensor) -> torch.Tensor:
         if self.has_any_delayed_scaling:
             self.float8_pre_forward(input)
         if isinstance(self.weight, Float8Tensor) or isinstance(input, Float8Tensor):

@@ -90,6 +90,7 @@ class Float8InferenceLinear(torch.nn.Linear):
             self._w_kb_key = key
         return self._w_kb
 
+    @torch._dynamo.disable  # the ctypes calls cannot be traced: under torch.compile this module runs outside the graph
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         if self.activation_casting == ActivationCasting.WEIGHT_ONLY:
             # the reference does not pass the bias on this branch either (inference.py:104-107)
