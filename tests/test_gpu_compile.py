@@ -114,6 +114,8 @@ def test_inductor_backend_if_it_is_usable_here(f8):
         got = _run(compiled, x, dy)
     except Exception as e:  # no code generator for this GPU in the installed torch: nothing of ours to test
         pytest.skip(f"inductor cannot generate code here: {type(e).__name__}")
-    # the float8 nodes are the same kernels; the compiler may fuse / re-associate its own bf16 pointwise code
+    # the float8 nodes are the same kernels, but the compiler fuses its own pointwise code (SiLU in fp32, one
+    # rounding), so the second layer sees inputs that differ in the last bf16 bit and a few of them fall on
+    # the other side of an fp8 rounding boundary: agreement is statistical, far above the float8 noise floor
     for a, b in zip(got, want):
-        assert torch.allclose(a.float(), b.float(), rtol=2e-2, atol=2e-2)
+        assert f8.float8_utils.compute_error(b.float(), a.float()).item() > 25
