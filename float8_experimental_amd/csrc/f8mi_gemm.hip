@@ -248,13 +248,9 @@ template <int AF, int BF, bool ALIGNED, int C_DT>
 static int launch_gemm3(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, const uint8_t* Bt, int64_t ldb, int M,
                         int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
                         int tiles_m, int tiles_n, int c_vec_ok) {
-    static bool attr_done = false;
+    static std::atomic<uint64_t> lds_allowed{0};
     auto kern = gemm_nt_kernel<AF, BF, ALIGNED, C_DT>;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
-        if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-        attr_done = true;
-    }
+    if (int rc = allow_big_lds(kern, GEMM_LDS, lds_allowed)) return rc;
     hipLaunchKernelGGL(kern, g, dim3(GEMM_THREADS), GEMM_LDS, stream, A, lda, Bt, ldb, M, N, K, sa, sb, C, ldc, bias,
                        tiles_m, tiles_n, c_vec_ok);
     return check_hip(hipGetLastError(), "gemm kernel launch");

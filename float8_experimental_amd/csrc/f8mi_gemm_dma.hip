@@ -214,13 +214,9 @@ template <int AF, int BF, int C_DT, bool ODD>
 static int launch_dma4(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb,
                        int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
                        int tiles_m, int tiles_n, int c_vec_ok) {
-    static bool attr_done = false;
+    static std::atomic<uint64_t> lds_allowed{0};
     auto kern = gemm_nt_dma_kernel<AF, BF, C_DT, ODD>;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, DMA_LDS);
-        if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-        attr_done = true;
-    }
+    if (int rc = allow_big_lds(kern, DMA_LDS, lds_allowed)) return rc;
     hipLaunchKernelGGL(kern, g, dim3(GEMM_THREADS), DMA_LDS, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias,
                        tiles_m, tiles_n, c_vec_ok);
     return check_hip(hipGetLastError(), "gemm (LDS-DMA) kernel launch");

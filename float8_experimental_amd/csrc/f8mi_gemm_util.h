@@ -1,6 +1,7 @@
 // Pieces shared by the two fp8 GEMM kernels (register-staged and LDS-DMA): tile constants,
 // fragment reads, output conversion and the C epilogue.
 #pragma once
+#include <atomic>
 #include <type_traits>
 
 #include "f8mi_common.h"
@@ -142,6 +143,21 @@ __device__ __forceinline__ void store_c_tile(v16f (&acc)[4][4], uint8_t* smem, i
             }
         }
     }
+}
+
+// Raises a kernel's dynamic LDS limit once per device (the attribute is per device, calls may come from any
+// host thread: a repeated call is harmless, a missing one is not).
+template <typename K>
+static int allow_big_lds(K kern, int bytes, std::atomic<uint64_t>& done_mask) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return check_hip(e, "hipGetDevice");
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done_mask.load(std::memory_order_acquire) & bit) return 0;
+    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    done_mask.fetch_or(bit, std::memory_order_release);
+    return 0;
 }
 
 // LDS-DMA kernel (f8mi_gemm_dma.hip).  Needs 16-byte aligned operands and strides and K % 64 == 0, K >= 384.
