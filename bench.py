@@ -180,6 +180,10 @@ def main():
             per_shape[name]["speedup_vs_bf16"] = per_shape[name]["bf16_ms"] / per_shape[name]["fp8_ms"]
         bf16_step = sum(v["bf16_ms"] for v in per_shape.values()) * 1e-3
 
+    # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
+    mfma_zero = _native.probe_mfma(False)
+    mfma_random = _native.probe_mfma(True)
+
     out = {
         "metric": "Float8Linear fwd+bwd TFLOP/s at LLaMa-2-70B shapes (1 GPU); cast GB/s",
         "value": flop_step / sec_step / 1e12,
@@ -211,6 +215,9 @@ def main():
             "launches": n_gemm,
             "avg_launch_ms": ms_gemm / max(n_gemm, 1),
             "flop_per_launch": flop_gemm / max(n_gemm, 1),
+            "mfma_only_zero_operands_TFLOP/s": mfma_zero,
+            "mfma_only_random_operands_TFLOP/s": mfma_random,
+            "frac_of_mfma_only_random": gemm_tflops / mfma_random if mfma_random > 0 else None,
         },
         "hbm_kernels": hbm,
         "per_shape": per_shape,

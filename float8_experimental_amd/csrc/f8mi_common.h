@@ -13,6 +13,7 @@ namespace f8mi {
 
 void set_error(const char* fmt, ...);
 int check_hip(hipError_t e, const char* what);
+int cu_count();  // compute units of the current device (f8mi_amax.hip)
 
 // Profiling brackets (no-ops unless f8mi_prof_enable(1) was called).
 struct ProfScope {

@@ -1,0 +1,92 @@
+// Measurement aid: what the fp8 matrix cores of this GPU sustain with no memory traffic at all.
+// A register-only loop of v_mfma_f32_16x16x128_f8f6f4 (the GEMM's instruction) over 64 accumulator
+// tiles per wave, one wave per SIMD on every CU.  On all-zero operands the loop runs at the clock limit;
+// on random fp8 bytes it runs into the power limit, which is the ceiling a real GEMM works under.
+#include <vector>
+
+#include "f8mi_common.h"
+
+namespace f8mi {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void mfma_probe_kernel(const int* __restrict__ in, float* __restrict__ out, int iters) {
+    v8i a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            a[i][j] = in[(threadIdx.x * 8 + j + i * 2048) & 65535];
+            b[i][j] = in[(threadIdx.x * 8 + j + i * 2048 + 17) & 65535];
+        }
+    v4f acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[i][j][e] = 0.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j & 3], a[i & 3], acc[i][j], 0, 0, 0, 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) s += acc[i][j][e];
+    out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+}  // namespace f8mi
+
+using namespace f8mi;
+
+extern "C" int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, size_t scratch_bytes, double* tflops, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    const int n_cu = cu_count();
+    const size_t need = 65536 * sizeof(int) + (size_t)n_cu * 256 * sizeof(float);
+    if (!scratch_dev || scratch_bytes < need || !tflops || iters < 1) { set_error("f8mi_probe_mfma: needs %zu bytes of device scratch, a result pointer and iters >= 1", need); return F8MI_ERR_INVALID_ARG; }
+    int* in = (int*)scratch_dev;
+    float* out = (float*)((char*)scratch_dev + 65536 * sizeof(int));
+    std::vector<int> h(65536, 0);
+    if (random_data) {
+        uint32_t state = 12345u;
+        for (auto& w : h) {
+            uint32_t v = 0;
+            for (int byte = 0; byte < 4; byte++) {
+                state = state * 1664525u + 1013904223u;
+                // sign random, exponent field 4..8 of 15 (finite, mid-range), mantissa random
+                const uint32_t e4m3 = ((state >> 24) & 0x80u) | ((4u + ((state >> 16) % 5u)) << 3) | ((state >> 8) & 7u);
+                v |= e4m3 << (8 * byte);
+            }
+            w = (int)v;
+        }
+    }
+    int rc = check_hip(hipMemcpyAsync(in, h.data(), 65536 * sizeof(int), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+    if (rc) return rc;
+    rc = check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+    if (rc) return rc;
+    hipEvent_t e0, e1;
+    if ((rc = check_hip(hipEventCreate(&e0), "hipEventCreate"))) return rc;
+    if ((rc = check_hip(hipEventCreate(&e1), "hipEventCreate"))) { (void)hipEventDestroy(e0); return rc; }
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(n_cu), dim3(256), 0, stream, in, out, iters / 8 + 1);  // warm-up
+    (void)hipEventRecord(e0, stream);
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(n_cu), dim3(256), 0, stream, in, out, iters);
+    (void)hipEventRecord(e1, stream);
+    rc = check_hip(hipEventSynchronize(e1), "hipEventSynchronize");
+    float ms = 0.f;
+    if (!rc) rc = check_hip(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc) return rc;
+    const double flop = 64.0 * 2 * 16 * 16 * 128 * (double)iters * 4 * n_cu;
+    *tflops = flop / (ms * 1e-3) / 1e12;
+    return F8MI_OK;
+}

@@ -498,3 +498,12 @@ def test_full_size_properties_llama70b_wo(nat):
     # grad_weight-shaped product from the transposed copies: (x^T x)[i][j], symmetric by construction
     g = nat.gemm_nt(x8t[:512], sx, x8t[:768], sx, torch.float32)
     torch.testing.assert_close(g[:, :512], g[:, :512].t(), rtol=1e-5, atol=1e-3)
+
+
+def test_mfma_probe_reports_a_sane_ceiling(nat):
+    """f8mi_probe_mfma: register-only MFMA loop; zeros run at the clock limit, random bytes below it."""
+    zero = nat.probe_mfma(False, iters=1000)
+    rnd = nat.probe_mfma(True, iters=1000)
+    assert 2000.0 < rnd <= zero * 1.02 and zero < 5300.0, (zero, rnd)
+    L = nat.lib()
+    assert L.f8mi_probe_mfma(0, 10, None, 0, None, None) != 0  # no scratch: refused on the host
