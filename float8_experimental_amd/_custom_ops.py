@@ -36,11 +36,17 @@ def _gemm(a8, sa, b8, sb, out_dtype, kb):
 @torch.library.custom_op("f8mi::linear_dynamic_fwd", mutates_args=())
 def linear_dynamic_fwd(x2: torch.Tensor, weight: torch.Tensor, need_dx: bool, need_dw: bool) -> Tuple[
         torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    """y = x2 W^T in fp8 with dynamic scales; also the transposed fp8 copies and scales backward needs.
+    """y = x2 W^T in fp8 with dynamic scales; also the fp8 copies and scales backward needs.
 
-    Returns (y, x8t, w8t, sx, sw); a copy that backward will not need is an empty tensor."""
+    Returns (y, xs, ws, sx, sw).  When every dimension allows it (``_native.tn_ok``) xs / ws are the forward's
+    own k-blocked operands (backward reads them transposed); otherwise they are the transposed copies, and
+    one that backward will not need is an empty tensor."""
     m, k = x2.shape
     n = weight.shape[0]
+    if _native.tn_ok(m, k, n):
+        x8, _, sx = _cast_dynamic(x2, e4m3_dtype, True, False, True, False)
+        w8, _, sw = _cast_dynamic(weight, e4m3_dtype, True, False, True, False)
+        return _native.gemm_nt_kb(x8, sx, w8, sw, x2.dtype), x8, w8, sx, sw
     kb_fwd, kb_dx, kb_dw = _native.kblock_ok(k), _native.kblock_ok(n), _native.kblock_ok(m)
     x8, x8t, sx = _cast_dynamic(x2, e4m3_dtype, True, need_dw, kb_fwd, kb_dw)
     w8, w8t, sw = _cast_dynamic(weight, e4m3_dtype, True, need_dx, kb_fwd, kb_dx)
@@ -53,29 +59,35 @@ def linear_dynamic_fwd(x2: torch.Tensor, weight: torch.Tensor, need_dx: bool, ne
 def _(x2, weight, need_dx, need_dw):
     m, k = x2.shape
     n = weight.shape[0]
-    kb_dx, kb_dw = _native.kblock_ok(n), _native.kblock_ok(m)
     f8 = lambda shape: torch.empty(shape, dtype=e4m3_dtype, device=x2.device)
     s = lambda: torch.empty((), dtype=torch.float32, device=x2.device)
-    return (torch.empty((m, n), dtype=x2.dtype, device=x2.device),
-            f8(_layout(k, m, kb_dw)) if need_dw else f8((0,)),
-            f8(_layout(k, n, kb_dx)) if need_dx else f8((0,)), s(), s())
+    y = torch.empty((m, n), dtype=x2.dtype, device=x2.device)
+    if _native.tn_ok(m, k, n):
+        return y, f8((k // _KB, m, _KB)), f8((k // _KB, n, _KB)), s(), s()
+    kb_dx, kb_dw = _native.kblock_ok(n), _native.kblock_ok(m)
+    return (y, f8(_layout(k, m, kb_dw)) if need_dw else f8((0,)), f8(_layout(k, n, kb_dx)) if need_dx else f8((0,)), s(), s())
 
 
 @torch.library.custom_op("f8mi::linear_dynamic_bwd", mutates_args=())
-def linear_dynamic_bwd(dy2: torch.Tensor, x8t: torch.Tensor, w8t: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor,
+def linear_dynamic_bwd(dy2: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor,
                        k: int, need_dx: bool, need_dw: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     """(dx, dw) = (dY W, dY^T x) in fp8, dY cast to e5m2 with a dynamic scale; an unneeded one is empty."""
     m, n = dy2.shape
+    empty = lambda: torch.empty(0, dtype=dy2.dtype, device=dy2.device)
+    if _native.tn_ok(m, k, n):
+        g8, _, sg = _cast_dynamic(dy2, e5m2_dtype, True, False, True, False)
+        dx = _native.gemm_kb_ex(g8, False, sg, ws, True, sw, dy2.dtype) if need_dx else empty()
+        dw = _native.gemm_kb_ex(g8, True, sg, xs, True, sx, dy2.dtype) if need_dw else empty()
+        return dx, dw
     kb_dx, kb_dw = _native.kblock_ok(n), _native.kblock_ok(m)
     g8, g8t, sg = _cast_dynamic(dy2, e5m2_dtype, need_dx, need_dw, kb_dx, kb_dw)
-    empty = lambda: torch.empty(0, dtype=dy2.dtype, device=dy2.device)
-    dx = _gemm(g8, sg, w8t, sw, dy2.dtype, kb_dx) if need_dx else empty()
-    dw = _gemm(g8t, sg, x8t, sx, dy2.dtype, kb_dw) if need_dw else empty()
+    dx = _gemm(g8, sg, ws, sw, dy2.dtype, kb_dx) if need_dx else empty()
+    dw = _gemm(g8t, sg, xs, sx, dy2.dtype, kb_dw) if need_dw else empty()
     return dx, dw
 
 
 @linear_dynamic_bwd.register_fake
-def _(dy2, x8t, w8t, sx, sw, k, need_dx, need_dw):
+def _(dy2, xs, ws, sx, sw, k, need_dx, need_dw):
     m, n = dy2.shape
     e = lambda shape: torch.empty(shape, dtype=dy2.dtype, device=dy2.device)
     return (e((m, k)) if need_dx else e((0,)), e((n, k)) if need_dw else e((0,)))

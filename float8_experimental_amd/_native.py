@@ -33,6 +33,7 @@ EXPORTS = (
     "f8mi_cast_layout",
     "f8mi_gemm_nt",
     "f8mi_gemm_nt_kb",
+    "f8mi_gemm_kb_ex",
     "f8mi_sync",
     "f8mi_delayed_init",
     "f8mi_prof_enable",
@@ -80,6 +81,8 @@ def lib() -> C.CDLL:
         L.f8mi_cast_layout.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, i32, vp, i32, fp, vp]
         L.f8mi_gemm_nt_kb.restype = i32
         L.f8mi_gemm_nt_kb.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
+        L.f8mi_gemm_kb_ex.restype = i32
+        L.f8mi_gemm_kb_ex.argtypes = [vp, i32, i32, vp, i32, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_nt.restype = i32
         L.f8mi_gemm_nt.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_sync.restype = i32
@@ -181,6 +184,12 @@ KB = 64          # depth of one block of the k-blocked operand layout
 KB_MIN_K = 384   # shortest contraction the k-blocked GEMM takes
 
 
+def tn_ok(*dims: int) -> bool:
+    """True if every dimension of a linear layer (tokens, in_features, out_features) allows the GEMMs to read
+    one k-blocked copy per tensor, transposed where needed (f8mi_gemm_kb_ex): multiples of 128, at least 384."""
+    return all(d % 128 == 0 and d >= KB_MIN_K for d in dims)
+
+
 def kblock_ok(k: int) -> bool:
     """True if a contraction of length k can use the k-blocked layout ([k/64][rows][64], see f8mi.h)."""
     return k % KB == 0 and k >= KB_MIN_K
@@ -253,6 +262,32 @@ def gemm_nt_kb(a_kb: torch.Tensor, a_scale: torch.Tensor, bt_kb: torch.Tensor, b
                                a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
                                bias.data_ptr() if bias is not None else None, _stream(a_kb))
     _check(rc, "f8mi_gemm_nt_kb")
+    return out
+
+
+def gemm_kb_ex(a_kb: torch.Tensor, a_transposed: bool, a_scale: torch.Tensor, bt_kb: torch.Tensor, b_transposed: bool,
+               b_scale: torch.Tensor, out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gemm_nt_kb whose operands may be given transposed (see f8mi_gemm_kb_ex).
+
+    ``a_kb`` is [k/64, m, 64] (not transposed) or [m/64, k, 64] (transposed: the k-blocked copy of the [k, m]
+    matrix, as the GEMM that contracts over m holds it); ``bt_kb`` likewise with n."""
+    _require_gpu(a_kb, "a_kb")
+    _require_gpu(bt_kb, "bt_kb")
+    for t in (a_kb, bt_kb):
+        assert t.dim() == 3 and t.shape[2] == KB and t.is_contiguous() and t.dtype in _F8, "k-blocked fp8 operands are contiguous [x/64, y, 64]"
+    m, k = (a_kb.shape[0] * KB, a_kb.shape[1]) if a_transposed else (a_kb.shape[1], a_kb.shape[0] * KB)
+    n, k2 = (bt_kb.shape[0] * KB, bt_kb.shape[1]) if b_transposed else (bt_kb.shape[1], bt_kb.shape[0] * KB)
+    assert k == k2, f"contraction lengths differ: {k} and {k2}"
+    for s in (a_scale, b_scale):
+        assert s.dtype == torch.float32 and s.numel() == 1 and s.device == a_kb.device, "scales: 1 fp32 element on the operands' device"
+    out = torch.empty((m, n), dtype=out_dtype, device=a_kb.device)
+    if bias is not None:
+        assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a_kb.device
+    _check_device(a_kb.device)
+    rc = lib().f8mi_gemm_kb_ex(a_kb.data_ptr(), _F8[a_kb.dtype], int(a_transposed), bt_kb.data_ptr(), _F8[bt_kb.dtype],
+                               int(b_transposed), m, n, k, a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(),
+                               _DT[out_dtype], max(n, 1), bias.data_ptr() if bias is not None else None, _stream(a_kb))
+    _check(rc, "f8mi_gemm_kb_ex")
     return out
 
 

@@ -344,3 +344,32 @@ extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_f
     return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
                            (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
 }
+
+extern "C" int f8mi_gemm_kb_ex(const void* a, int a_fmt, int a_transposed, const void* bt, int b_fmt, int b_transposed,
+                               int64_t m, int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c,
+                               int c_dtype, int64_t ldc, const void* bias_dev, void* stream_) {
+    if (!a_transposed && !b_transposed)
+        return f8mi_gemm_nt_kb(a, a_fmt, bt, b_fmt, m, n, k, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, stream_);
+    hipStream_t stream = (hipStream_t)stream_;
+    if (a_transposed && !b_transposed) { set_error("f8mi_gemm_kb_ex: a transposed with bt not transposed is not built (swap the operands and transpose c)"); return F8MI_ERR_UNSUPPORTED; }
+    if (m < 0 || n < 0 || k < 0 || ldc < n) { set_error("f8mi_gemm_kb_ex: bad shape m=%lld n=%lld k=%lld ldc=%lld", (long long)m, (long long)n, (long long)k, (long long)ldc); return F8MI_ERR_INVALID_ARG; }
+    if (a_fmt < 0 || a_fmt > 1 || b_fmt < 0 || b_fmt > 1 || c_dtype < 0 || c_dtype > 2) { set_error("f8mi_gemm_kb_ex: unknown format/dtype code"); return F8MI_ERR_INVALID_ARG; }
+    if (k % 128 != 0 || k < 384) { set_error("f8mi_gemm_kb_ex: transposed operands need k %% 128 == 0 and k >= 384 (k=%lld)", (long long)k); return F8MI_ERR_UNSUPPORTED; }
+    if (n % 64 != 0 || (a_transposed && m % 64 != 0)) { set_error("f8mi_gemm_kb_ex: a transposed operand needs its row count to be a multiple of 64 (m=%lld n=%lld)", (long long)m, (long long)n); return F8MI_ERR_UNSUPPORTED; }
+    if (m == 0 || n == 0) return F8MI_OK;
+    if (!a || !bt || !c || !scale_a_dev || !scale_b_dev) { set_error("f8mi_gemm_kb_ex: null pointer"); return F8MI_ERR_INVALID_ARG; }
+    if ((uintptr_t)a % 16 != 0 || (uintptr_t)bt % 16 != 0) { set_error("f8mi_gemm_kb_ex: operands must be 16-byte aligned"); return F8MI_ERR_UNSUPPORTED; }
+    if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff - BK || k * 64 * 4 > 0x7fffffffLL) { set_error("f8mi_gemm_kb_ex: dimension too large"); return F8MI_ERR_UNSUPPORTED; }
+    const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    if (tiles_m * tiles_n > 0x7fffffff) { set_error("f8mi_gemm_kb_ex: too many tiles"); return F8MI_ERR_UNSUPPORTED; }
+    const int64_t csz = c_dtype == F8MI_FP32 ? 4 : 2;
+    const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
+    dim3 g((unsigned)(tiles_m * tiles_n));
+    ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
+    // a transposed operand: 64 bytes between contraction rows, k * 64 between blocks of 64 rows
+    if (a_transposed)
+        return launch_gemm_dma16_tt(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, k * 64, (const uint8_t*)bt, 64, k * 64, (int)m, (int)n,
+                                    (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    return launch_gemm_dma16_nt(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, k * 64, (int)m, (int)n,
+                                (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+}

@@ -1,0 +1,417 @@
+// Implementation of the 16x16x128 LDS-DMA GEMM kernel, shared by the translation units that instantiate it
+// for normal and transposed operands (f8mi_gemm_dma16*.hip).
+#pragma once
+#include "f8mi_gemm_util.h"
+
+namespace f8mi {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int SLAB_BYTES = 256 * 128;   // one operand, one step
+constexpr int HALF_BYTES = 256 * 64;    // one 64-deep unit of it
+constexpr int NSLAB_A = 3, NSLAB_B = 2;
+constexpr int DMA16_LDS = (NSLAB_A + NSLAB_B) * SLAB_BYTES;  // 160 KB
+static_assert(DMA16_LDS >= EPI_BYTES, "the C staging tile reuses the slabs");
+
+__device__ __forceinline__ void dma16b(const uint8_t* base, uint32_t voff, uint32_t lds_addr) {
+    // M0 carries the LDS address; one wait state between the scalar write of M0 and its use
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds_addr) : "memory");
+}
+
+// acc += first (16 rows x 128 k, format F1) * second^T (16 rows x 128 k, format F2); formats 0 = e4m3, 1 = e5m2.
+// Written as an instruction so that the accumulator is an AGPR tuple updated in place: left to the
+// register allocator, a quarter of the 64 accumulators ends up commuting between register files.
+// The compiler does not know this is a matrix instruction: callers keep the required distance
+// between the last one and the first read of an accumulator themselves.
+template <int F1, int F2>
+__device__ __forceinline__ void mfma16(v4f& acc, const v8i& first, const v8i& second) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:%3 blgp:%4" : "+a"(acc) : "v"(first), "v"(second), "n"(F1), "n"(F2));
+}
+// acc = first * second^T: the first step of a tile starts from the constant 0 instead of zeroed
+// registers (a register written by an ordinary vector instruction must not be read by a matrix
+// instruction right away, and nothing here would keep the compiler from placing the two back to back).
+template <int F1, int F2>
+__device__ __forceinline__ void mfma16_first(v4f& acc, const v8i& first, const v8i& second) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:%3 blgp:%4" : "=a"(acc) : "v"(first), "v"(second), "n"(F1), "n"(F2));
+}
+
+// Scales the 8 x 8 tiles of 16 x 16 accumulators, adds the bias, converts and writes C.
+// acc[tj][ti] as left by MFMA(first = Bt rows, second = A rows): lane holds row ti*16 + lane%16
+// and the four columns tj*16 + 4*(lane/16) + e of its wave's 128 x 128 quarter.
+template <int C_DT>
+__device__ __forceinline__ void store_c_tile16(v4f (&acc)[8][8], uint8_t* smem, int m0, int n0, int M, int N,
+                                               const float* __restrict__ sa_dev, const float* __restrict__ sb_dev,
+                                               void* __restrict__ C, int64_t ldc, const void* __restrict__ bias,
+                                               int c_vec_ok) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
+    const int lm = lane & 15, lq = lane >> 4;
+    const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
+
+    if constexpr (C_DT == F8MI_FP32) {
+        float* Cf = (float*)C;
+#pragma unroll
+        for (int tj = 0; tj < 8; tj++) {
+            const int col = wcol0 + tj * 16 + 4 * lq;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (col + r < N) bv[r] = load_bias<C_DT>(bias, col + r);
+            }
+#pragma unroll
+            for (int ti = 0; ti < 8; ti++) {
+                const int row = wrow0 + ti * 16 + lm;
+                if (row >= M || col >= N) continue;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] = acc[tj][ti][r] * inv + bv[r];
+                float* dst = Cf + (int64_t)row * ldc + col;
+                if (c_vec_ok && col + 4 <= N) {
+                    *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (col + r < N) dst[r] = v[r];
+                }
+            }
+        }
+    } else {
+        lds_barrier();  // all waves are done with the operand slabs before they become the output staging area
+        uint8_t* ep = smem + wave * (128 * EPI_PITCH);
+#pragma unroll
+        for (int tj = 0; tj < 8; tj++) {
+            const int cl = tj * 16 + 4 * lq;  // column inside the wave's 128
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (wcol0 + cl + r < N) bv[r] = load_bias<C_DT>(bias, wcol0 + cl + r);
+            }
+#pragma unroll
+            for (int ti = 0; ti < 8; ti++) {
+                const float v0 = acc[tj][ti][0] * inv + bv[0];
+                const float v1 = acc[tj][ti][1] * inv + bv[1];
+                const float v2 = acc[tj][ti][2] * inv + bv[2];
+                const float v3 = acc[tj][ti][3] * inv + bv[3];
+                *(uint2*)(ep + (ti * 16 + lm) * EPI_PITCH + cl * 2) = make_uint2(pack2<C_DT>(v0, v1), pack2<C_DT>(v2, v3));
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own wave's tile only: no workgroup barrier needed
+        uint16_t* Ch = (uint16_t*)C;
+        const int chunk = lane & 15, rsub = lane >> 4;
+        const int col = wcol0 + chunk * 8;
+#pragma unroll 4
+        for (int it = 0; it < 32; it++) {
+            const int rl = it * 4 + rsub;
+            const int row = wrow0 + rl;
+            const uint4 v = *(const uint4*)(ep + rl * EPI_PITCH + chunk * 16);
+            if (row < M && col < N) {
+                uint16_t* dst = Ch + (int64_t)row * ldc + col;
+                if (c_vec_ok && col + 8 <= N) {
+                    *(uint4*)dst = v;
+                } else {
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++)
+                        if (col + i < N) dst[i] = (uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+                }
+            }
+        }
+    }
+}
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+// Four transpose reads = the 32 contraction bytes of one lane's MFMA operand (rows k0 + 8t .. + 7, t = 0..3, of
+// the lane's column): in every group of 16 lanes, lane i receives byte i%8 of the 8 bytes addressed by lanes
+// 2b + i/8 (b = 0..7); callers point lane j at (row k0 + j/2, column n0 + 8*(j%2)), so lane i gets column n0 + i.
+__device__ __forceinline__ v8i read_frag_tr(const uint8_t* p) {
+    typedef __attribute__((address_space(3))) v2i* lds_v2i;
+    const v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p));
+    const v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 2048));
+    const v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 4096));
+    const v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(p + 6144));
+    return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
+}
+
+// f(k) of the transposed-slab swizzle: the 16-byte slot c of contraction row k sits at slot c ^ f(k).  One
+// transpose read touches rows 8t..8t+7 of two 32-row quarters per 32 lanes; f makes those 16 rows hit 16
+// different slots.
+__device__ __forceinline__ int tr_swizzle(int k) { return (k & 7) | (((k >> 5) & 1) << 3); }
+
+// ODD (from the host): the number of steps K/128 is odd.
+// A_TR / B_TR: the operand is given "transposed": its memory holds the matrix [contraction][rows] (the layout
+// in which another GEMM contracts over `rows`), a slab is 128 contraction rows x 256 row-bytes, and fragments
+// are built with ds_read_b64_tr_b8.  For such an operand lda / ldb is the byte distance between contraction
+// rows (64 when k-blocked over `rows`, the row stride when row-major) and a_unit / b_unit the distance between
+// blocks of 64 rows (contraction length * 64 when k-blocked, 64 when row-major).
+template <int AF, int BF, int C_DT, bool ODD, bool A_TR, bool B_TR>
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
+    const uint8_t* __restrict__ A, int64_t lda, int64_t a_unit, const uint8_t* __restrict__ Bt, int64_t ldb, int64_t b_unit,
+    int M, int N, int K, const float* __restrict__ sa_dev, const float* __restrict__ sb_dev, void* __restrict__ C,
+    int64_t ldc, const void* __restrict__ bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    // lda / ldb: bytes from one operand row to the next; a_unit / b_unit: bytes from one 64-deep unit
+    // to the next.  Row-major operands: (row stride, 64); k-blocked [K/64][rows][64]: (64, rows*64).
+
+    // ---- which tile (same walk as the other kernels)
+    int lid = blockIdx.x;
+    const int npid = gridDim.x;
+    if (npid % NUM_XCD == 0) lid = (lid % NUM_XCD) * (npid / NUM_XCD) + lid / NUM_XCD;
+    constexpr int GROUP = 4;  // tile rows per walk group: an XCD's 32 workgroups then hold 4 x 8 neighbouring tiles
+    const int width = GROUP * tiles_n;
+    const int group = lid / width;
+    const int first_m = group * GROUP;
+    const int gsz = min(tiles_m - first_m, GROUP);
+    const int tm = first_m + (lid % width) % gsz;
+    const int tn = (lid % width) / gsz;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- DMA addressing.
+    // Normal operand: instruction j = wave*4 + i of a slab half covers tile rows 16j .. 16j+15; lane l fetches
+    // row 16j + l/4, 16-byte piece (l%4) ^ ((l/16) % 4) (the swizzle, applied on the global side).
+    // Transposed operand: instruction j = wave*8 + d covers contraction rows 4j .. 4j+3 of the slab, 256 bytes
+    // (16 slots) each; lane l fetches row 4j + l/16, the slot that belongs at position l%16: (l%16) ^ f(row).
+    const uint32_t lds_u32 = (uint32_t)(uintptr_t)smem;
+    uint32_t a_voff[A_TR ? 8 : 4], b_voff[B_TR ? 8 : 4];
+    const uint8_t* a_ptr;  // first byte of the next step to be fetched
+    const uint8_t* b_ptr;
+    int64_t a_step, b_step;  // bytes from one step's data to the next
+    if constexpr (A_TR) {
+#pragma unroll
+        for (int d = 0; d < 8; d++) {
+            const int rowl = 4 * (wave * 8 + d) + (lane >> 4);
+            const int c = (lane & 15) ^ tr_swizzle(rowl);
+            const int blk = min(m0 / 64 + (c >> 2), M / 64 - 1) - m0 / 64;  // blocks past the edge re-read the last one
+            a_voff[d] = (uint32_t)(rowl * lda + blk * a_unit) + (c & 3) * 16;
+        }
+        a_ptr = A + (int64_t)(m0 / 64) * a_unit;
+        a_step = 128 * lda;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int r = (wave * 4 + i) * 16 + (lane >> 2);
+            a_voff[i] = (uint32_t)(min(r, M - 1 - m0) * lda) + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);  // rows past the edge re-read the last row
+        }
+        a_ptr = A + (int64_t)m0 * lda;
+        a_step = 2 * a_unit;
+    }
+    if constexpr (B_TR) {
+#pragma unroll
+        for (int d = 0; d < 8; d++) {
+            const int rowl = 4 * (wave * 8 + d) + (lane >> 4);
+            const int c = (lane & 15) ^ tr_swizzle(rowl);
+            const int blk = min(n0 / 64 + (c >> 2), N / 64 - 1) - n0 / 64;
+            b_voff[d] = (uint32_t)(rowl * ldb + blk * b_unit) + (c & 3) * 16;
+        }
+        b_ptr = Bt + (int64_t)(n0 / 64) * b_unit;
+        b_step = 128 * ldb;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int r = (wave * 4 + i) * 16 + (lane >> 2);
+            b_voff[i] = (uint32_t)(min(r, N - 1 - n0) * ldb) + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
+        }
+        b_ptr = Bt + (int64_t)n0 * ldb;
+        b_step = 2 * b_unit;
+    }
+    uint32_t a_dst = 0, b_dst = 0;  // LDS address of the slabs being refilled
+    // DMA d = 0..7 of this wave's share of a slab
+    auto issue_a = [&](int d) __attribute__((always_inline)) {
+        if constexpr (A_TR) dma16b(a_ptr, a_voff[d], a_dst + (wave * 8 + d) * 1024);
+        else dma16b(d < 4 ? a_ptr : a_ptr + a_unit, a_voff[d & 3], a_dst + wave * 4096 + (d >> 2) * HALF_BYTES + (d & 3) * 1024);
+        if (d == 7) a_ptr += a_step;
+    };
+    auto issue_b = [&](int d) __attribute__((always_inline)) {
+        if constexpr (B_TR) dma16b(b_ptr, b_voff[d], b_dst + (wave * 8 + d) * 1024);
+        else dma16b(d < 4 ? b_ptr : b_ptr + b_unit, b_voff[d & 3], b_dst + wave * 4096 + (d >> 2) * HALF_BYTES + (d & 3) * 1024);
+        if (d == 7) b_ptr += b_step;
+    };
+
+    // ---- fragment addressing.
+    // Normal operand: lane -> tile row lane % 16, k quarter lane / 16 (32 bytes: half q/2, pieces 2(q%2), 2(q%2)+1).
+    // Transposed operand: lane j of a 16-lane group q addresses contraction row 32q + 8t + j/2 (t-th read),
+    // byte column tile*16 + 8*(j%2) of the wave's 128 columns, through the slot swizzle.
+    const int frow = lane & 15, fq = lane >> 4;
+    const int fsw = (frow >> 2) & 3;
+    const int f_off0 = (fq >> 1) * HALF_BYTES + frow * 64 + ((((fq & 1) * 2 + 0) ^ fsw) << 4);
+    const int f_off1 = (fq >> 1) * HALF_BYTES + frow * 64 + ((((fq & 1) * 2 + 1) ^ fsw) << 4);
+    const int tr_f = tr_swizzle(32 * fq + (frow >> 1));  // the same for all four reads of a lane
+    int a_tr_off[A_TR ? 8 : 1], b_tr_off[B_TR ? 8 : 1];
+    if constexpr (A_TR) {
+        const int base = (32 * fq + (frow >> 1)) * 256 + 128 * (wm ^ (tr_f >> 3)) + 8 * (frow & 1);
+#pragma unroll
+        for (int x = 0; x < 8; x++) a_tr_off[x] = base + ((x ^ (tr_f & 7)) << 4);
+    }
+    if constexpr (B_TR) {
+        const int base = (32 * fq + (frow >> 1)) * 256 + 128 * (wn ^ (tr_f >> 3)) + 8 * (frow & 1);
+#pragma unroll
+        for (int x = 0; x < 8; x++) b_tr_off[x] = base + ((x ^ (tr_f & 7)) << 4);
+    }
+    const int a_frag_base = (wm * 128) * 64;
+    const int b_frag_base = (wn * 128) * 64;
+    auto frag_a = [&](const uint8_t* slab, int ti) __attribute__((always_inline)) {
+        if constexpr (A_TR) {
+            return read_frag_tr(slab + a_tr_off[ti]);
+        } else {
+            const uint8_t* p = slab + a_frag_base + ti * 16 * 64;
+            return read_frag(p + f_off0, p + f_off1);
+        }
+    };
+    auto frag_b = [&](const uint8_t* slab, int tj) __attribute__((always_inline)) {
+        if constexpr (B_TR) {
+            return read_frag_tr(slab + b_tr_off[tj]);
+        } else {
+            const uint8_t* p = slab + b_frag_base + tj * 16 * 64;
+            return read_frag(p + f_off0, p + f_off1);
+        }
+    };
+
+    v4f acc[8][8];  // first written by step 0
+
+    v8i fb[2][8];  // [step parity][n tile]
+    v8i fa[2];     // rolling: group ti multiplies fa[ti & 1] while fa[(ti + 1) & 1] is being fetched
+
+    // ---- prologue: steps 0 and 1 (A into slabs 0, 1; Bt into slabs 3, 4), wait for step 0,
+    // first fragments; a second barrier before step 0 refills the Bt slab just read.
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        a_dst = lds_u32 + s * SLAB_BYTES;
+        b_dst = lds_u32 + (NSLAB_A + s) * SLAB_BYTES;
+#pragma unroll
+        for (int d = 0; d < 8; d++) issue_a(d);
+#pragma unroll
+        for (int d = 0; d < 8; d++) issue_b(d);
+    }
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    lds_barrier();
+#pragma unroll
+    for (int x = 0; x < 8; x++) fb[0][x] = frag_b(smem + NSLAB_A * SLAB_BYTES, x);
+    fa[0] = frag_a(smem, 0);
+    lds_barrier();
+
+    // One step t.  P: parity of t.  MODE 0: steps t+1 and t+2 exist (refills the slabs freed at this
+    // step's start with step t+2); 1: last but one (nothing left to fetch); 2: last step; 3: step 0 (as 0,
+    // and the accumulators start from zero).
+    int a_slab = 0;  // slab of A of this step; step t+2 goes to the slab before it in the rotation
+    auto step = [&](auto parity, auto mode) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value;
+        constexpr bool FIRST = decltype(mode)::value == 3;
+        constexpr int MODE = FIRST ? 0 : decltype(mode)::value;
+        const int a_next = a_slab + 1 == NSLAB_A ? 0 : a_slab + 1;
+        const int a_free = a_next + 1 == NSLAB_A ? 0 : a_next + 1;  // held step t-1
+        const uint8_t* a_cur = smem + a_slab * SLAB_BYTES;
+        const uint8_t* a_nxt = smem + a_next * SLAB_BYTES;
+        const uint8_t* b_nxt = smem + (NSLAB_A + (P ^ 1)) * SLAB_BYTES;
+        if (MODE == 0) {
+            a_dst = lds_u32 + a_free * SLAB_BYTES;
+            b_dst = lds_u32 + (NSLAB_A + P) * SLAB_BYTES;  // Bt of this step: already in registers
+        }
+        // Everything that is not an MFMA sits in a fixed slot between two MFMAs (each keeps the matrix
+        // core busy for 32 cycles): one fragment (two 16-byte LDS reads) or one DMA at a time.
+#pragma unroll
+        for (int ti = 0; ti < 8; ti++) {
+            if (ti == 6 && MODE < 2) {
+                // this wave's DMAs of step t+1 have landed (the 12 of step t+2 issued so far may be in flight) ...
+                if (MODE == 0) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                asm volatile("s_barrier" ::: "memory");  // ... and so have everybody's; no LDS hazard here, so no wait on LDS reads
+            }
+#pragma unroll
+            for (int tj = 0; tj < 8; tj++) {
+                if (tj == 0 && ti < 7) fa[(ti + 1) & 1] = frag_a(a_cur, ti + 1);
+                if (tj == 0 && ti == 7 && MODE < 2) fa[0] = frag_a(a_nxt, 0);
+                if (MODE < 2 && ti >= 6 && (tj & 1) == 1) fb[P ^ 1][(ti - 6) * 4 + (tj >> 1)] = frag_b(b_nxt, (ti - 6) * 4 + (tj >> 1));
+                if (FIRST) mfma16_first<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
+                else mfma16<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
+                F8MI_SCHED_FENCE();
+                if (MODE == 0 && (tj & 3) == 0) {
+                    // 16 DMAs over the 64 MFMAs, one after every fourth: A slab first, then Bt.  (Packed into
+                    // the first half of the step they cost 3 % more time: the four waves share one load unit.)
+                    const int d = ti * 2 + (tj >> 2);
+                    if (d < 8) issue_a(d);
+                    else issue_b(d - 8);
+                    F8MI_SCHED_FENCE();
+                }
+            }
+        }
+        if (MODE < 2) lds_barrier();  // step boundary: everybody is done with A of step t and has Bt of step t+1 in registers
+        a_slab = a_next;
+    };
+
+    constexpr std::integral_constant<int, 0> c0{};
+    constexpr std::integral_constant<int, 1> c1{};
+    constexpr std::integral_constant<int, 2> c2{};
+
+    constexpr std::integral_constant<int, 3> c3{};
+    const int n_steady = K / 128 - 2;  // steps that fetch: >= 1 (host); ODD <=> odd
+    step(c0, c3);
+    if constexpr (ODD) {
+        for (int s = 1; s < n_steady; s += 2) {
+            step(c1, c0);
+            step(c0, c0);
+        }
+        step(c1, c1);
+        step(c0, c2);
+    } else {
+        step(c1, c0);
+        for (int s = 2; s < n_steady; s += 2) {
+            step(c0, c0);
+            step(c1, c0);
+        }
+        step(c0, c1);
+        step(c1, c2);
+    }
+    // the last MFMAs are still in the pipeline (8 passes): keep the accumulator reads away from them
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    store_c_tile16<C_DT>(acc, smem, m0, n0, M, N, sa_dev, sb_dev, C, ldc, bias, c_vec_ok);
+}
+
+template <int AF, int BF, int C_DT, bool ODD, bool A_TR, bool B_TR>
+static int launch16_4(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb,
+                      int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
+                      const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    static std::atomic<uint64_t> lds_allowed{0};
+    auto kern = gemm_nt_dma16_kernel<AF, BF, C_DT, ODD, A_TR, B_TR>;
+    if (int rc = allow_big_lds(kern, DMA16_LDS, lds_allowed)) return rc;
+    hipLaunchKernelGGL(kern, g, dim3(GEMM_THREADS), DMA16_LDS, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C,
+                       ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return check_hip(hipGetLastError(), "gemm (LDS-DMA, 16x16x128) kernel launch");
+}
+
+template <int AF, int BF, int C_DT, bool A_TR, bool B_TR>
+static int launch16_3(dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb,
+                      int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
+                      const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    if ((K / 128) & 1) return launch16_4<AF, BF, C_DT, true, A_TR, B_TR>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch16_4<AF, BF, C_DT, false, A_TR, B_TR>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+}
+
+template <int AF, int BF, bool A_TR, bool B_TR>
+static int launch16_2(int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt,
+                      int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
+                      const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    if (c_dtype == F8MI_BF16) return launch16_3<AF, BF, F8MI_BF16, A_TR, B_TR>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (c_dtype == F8MI_FP16) return launch16_3<AF, BF, F8MI_FP16, A_TR, B_TR>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch16_3<AF, BF, F8MI_FP32, A_TR, B_TR>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+}
+
+template <bool A_TR, bool B_TR>
+static int launch_gemm_dma16_t(int a_fmt, int b_fmt, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
+                      const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb,
+                      void* C, int64_t ldc, const void* bias, int tiles_m, int tiles_n, int c_vec_ok) {
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch16_2<0, 0, A_TR, B_TR>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch16_2<1, 0, A_TR, B_TR>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch16_2<0, 1, A_TR, B_TR>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+    return launch16_2<1, 1, A_TR, B_TR>(c_dtype, g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, tiles_n, c_vec_ok);
+}
+
+}  // namespace f8mi

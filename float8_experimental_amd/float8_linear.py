@@ -91,9 +91,12 @@ def _gemm(a8, sa, b8, sb, out_dtype, kb: bool):
 class _float8_linear_fn(torch.autograd.Function):
     """y = x W^T with every matmul of forward and backward in fp8 (no bias).
 
-    Each of the three GEMMs contracts a different dimension (in_features, out_features,
-    tokens); where that length allows it (a multiple of 64, at least 384) both of its
-    operands are produced k-blocked by the cast kernel, which is the GEMM's fastest input.
+    Each of the three GEMMs contracts a different dimension (in_features, out_features, tokens).
+    When all three are multiples of 128 (and at least 384) each tensor is cast ONCE, k-blocked over
+    its own last dimension, and the two GEMMs that use it read that one copy -- as it is where its last
+    dimension is contracted, through LDS transpose loads where it is not (``f8mi_gemm_kb_ex``): no
+    transposed fp8 copies exist.  Otherwise the cast writes the tensor and its transpose, each k-blocked
+    where its GEMM's contraction allows it (a multiple of 64, at least 384) and row-major where not.
     """
 
     @staticmethod
@@ -104,34 +107,50 @@ class _float8_linear_fn(torch.autograd.Function):
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         emulate = mod.linear_mm_config.output.emulate
         emulate_bw = mod.linear_mm_config.grad_input.emulate or mod.linear_mm_config.grad_weight.emulate
-        kb_fwd = not emulate and _native.kblock_ok(k)      # y = x W^T contracts in_features
-        kb_dx = not emulate_bw and _native.kblock_ok(n)    # dx = dy W contracts out_features
-        kb_dw = not emulate_bw and _native.kblock_ok(m)    # dw = dy^T x contracts tokens
         dl = mod._delayed_buffers
-        x8, x8t, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, need_dw, kb_fwd, kb_dw)
-        w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx, kb_fwd, kb_dx)
-        if emulate:
-            y = mm_float8_emulated(x8, sx, w8.t(), sw, x.dtype)
+        tn = not emulate and not emulate_bw and _native.tn_ok(m, k, n)
+        if tn:
+            x8, _, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, False, True, False)
+            w8, _, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, False, True, False)
+            y = _native.gemm_nt_kb(x8, sx, w8, sw, x.dtype)
+            ctx.kb = None
+            ctx.save_for_backward(x8, w8, sx, sw)
         else:
-            y = _gemm(x8, sx, w8, sw, x.dtype, kb_fwd)
+            kb_fwd = not emulate and _native.kblock_ok(k)      # y = x W^T contracts in_features
+            kb_dx = not emulate_bw and _native.kblock_ok(n)    # dx = dy W contracts out_features
+            kb_dw = not emulate_bw and _native.kblock_ok(m)    # dw = dy^T x contracts tokens
+            x8, x8t, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, need_dw, kb_fwd, kb_dw)
+            w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx, kb_fwd, kb_dx)
+            if emulate:
+                y = mm_float8_emulated(x8, sx, w8.t(), sw, x.dtype)
+            else:
+                y = _gemm(x8, sx, w8, sw, x.dtype, kb_fwd)
+            ctx.kb = (kb_dx, kb_dw)
+            ctx.save_for_backward(x8t, w8t, sx, sw)
         ctx.mod = mod
         ctx.is_amax_initialized = is_amax_initialized
         ctx.x_shape = x.shape
-        ctx.kb = (kb_dx, kb_dw)
-        ctx.save_for_backward(x8t, w8t, sx, sw)
         return y.reshape(*x.shape[:-1], n)
 
     @staticmethod
     def backward(ctx, dy):
-        x8t, w8t, sx, sw = ctx.saved_tensors
         mod = ctx.mod
-        kb_dx, kb_dw = ctx.kb
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         dy2 = dy.reshape(-1, dy.shape[-1])
-        g8, g8t, sg = _cast_for_gemm(dy2, e5m2_dtype, mod._delayed_buffers("grad_output"), ctx.is_amax_initialized,
-                                     need_dx, need_dw, kb_dx, kb_dw)
-        emulate = mod.linear_mm_config.grad_input.emulate
+        dlg = mod._delayed_buffers("grad_output")
         dx = dw = None
+        if ctx.kb is None:  # one copy per tensor: x8 [K/64, M, 64], w8 [K/64, N, 64], g8 [N/64, M, 64]
+            x8, w8, sx, sw = ctx.saved_tensors
+            g8, _, sg = _cast_for_gemm(dy2, e5m2_dtype, dlg, ctx.is_amax_initialized, True, False, True, False)
+            if need_dx:  # grad_input = dY @ W: dY as it is, W read transposed
+                dx = _native.gemm_kb_ex(g8, False, sg, w8, True, sw, dy.dtype).reshape(ctx.x_shape)
+            if need_dw:  # grad_weight = dY^T @ x: both read transposed
+                dw = _native.gemm_kb_ex(g8, True, sg, x8, True, sx, dy.dtype)
+            return dx, dw, None, None
+        x8t, w8t, sx, sw = ctx.saved_tensors
+        kb_dx, kb_dw = ctx.kb
+        g8, g8t, sg = _cast_for_gemm(dy2, e5m2_dtype, dlg, ctx.is_amax_initialized, need_dx, need_dw, kb_dx, kb_dw)
+        emulate = mod.linear_mm_config.grad_input.emulate
         if need_dx:  # grad_input = dY @ W          [M,N] x [N,K]
             if emulate:
                 dx = mm_float8_emulated(g8, sg, w8t.t(), sw, dy.dtype)

@@ -145,6 +145,18 @@ int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t
                     const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
                     const void* bias_dev, void* stream);
 
+/* f8mi_gemm_nt_kb with operands that may be given transposed, so that one k-blocked copy of a tensor serves
+ * both GEMMs that use it (no transposed fp8 copies at all):
+ *   a, a_transposed = 0: [k/64][m][64] as above;  = 1: [m/64][k][64], i.e. the matrix [k][m] k-blocked over m
+ *   bt likewise with n.
+ * Forward x*W^T takes (0, 0); grad_input dY*W takes a = dY8 [n_out/64][tokens][64] (0) and bt = the forward's
+ * W8 [k_in/64][n_out][64] (1); grad_weight dY^T*x takes a = that dY8 (1) and bt = the forward's x8 (1).
+ * (1, 0) is not built.  Transposed operands need k % 128 == 0, k >= 384 and the operand's row count (m or n)
+ * to be a multiple of 64.  Same result bits as f8mi_gemm_nt on the row-major operands. */
+int f8mi_gemm_kb_ex(const void* a, int a_fmt, int a_transposed, const void* bt, int b_fmt, int b_transposed, int64_t m,
+                    int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
+                    int64_t ldc, const void* bias_dev, void* stream);
+
 /* One (layer, tensor) row of the delayed-scaling bookkeeping; all device pointers. */
 typedef struct f8mi_sync_entry {
     float* amax;    /* [1]        fp8_amax_*          */

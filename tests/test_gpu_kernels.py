@@ -361,6 +361,29 @@ def test_gemm_kblocked_equals_row_major_bitwise(nat, m, n, k):
         assert torch.equal(got, want), (m, n, k, out_dt)
 
 
+@pytest.mark.parametrize("m,n,k", [(256, 256, 384), (320, 192, 512), (64, 128, 640), (704, 448, 1024), (512, 256, 8192),
+                                   (16384 // 8, 1024, 2048)])
+def test_gemm_with_transposed_operands_equals_row_major_bitwise(nat, m, n, k):
+    """f8mi_gemm_kb_ex: Bt, or A and Bt, given as the k-blocked copy of the transposed matrix (what the other
+    GEMMs of a linear layer hold), read with LDS transpose loads: identical bits to the row-major GEMM."""
+    a = _rand_fp8((m, k), torch.float8_e5m2, m + k + 5, 4.0).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e4m3fn, n + k + 6, 4.0).to(DEV)
+    sa, sb = torch.tensor(3.0, device=DEV), torch.tensor(0.5, device=DEV)
+    a_tr = _to_kb(a.view(torch.uint8).t().contiguous().view(a.dtype))    # [m/64, k, 64]
+    bt_tr = _to_kb(bt.view(torch.uint8).t().contiguous().view(bt.dtype))  # [n/64, k, 64]
+    bias = (torch.randn(n) * 3).to(torch.bfloat16).to(DEV)
+    for out_dt, b in ((torch.bfloat16, bias), (torch.float32, None)):
+        want = nat.gemm_nt(a, sa, bt, sb, out_dt, bias=b)
+        got = nat.gemm_kb_ex(_to_kb(a), False, sa, bt_tr, True, sb, out_dt, bias=b)
+        assert torch.equal(got, want), (m, n, k, out_dt, "bt transposed")
+        got = nat.gemm_kb_ex(a_tr, True, sa, bt_tr, True, sb, out_dt, bias=b)
+        assert torch.equal(got, want), (m, n, k, out_dt, "both transposed")
+        got = nat.gemm_kb_ex(_to_kb(a), False, sa, _to_kb(bt), False, sb, out_dt, bias=b)
+        assert torch.equal(got, want)
+    with pytest.raises(nat.Float8NativeError):
+        nat.gemm_kb_ex(a_tr, True, sa, _to_kb(bt), False, sb, torch.bfloat16)
+
+
 def test_gemm_kblocked_refuses_short_or_ragged_k(nat):
     s1 = torch.ones((), device=DEV)
     for k in (64, 320):

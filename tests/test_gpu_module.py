@@ -202,10 +202,13 @@ def test_fused_forward_equals_the_composed_reference_pipeline(f8, scaling):
 
 
 @pytest.mark.parametrize("scaling", [("dyn", "dyn", "dyn"), ("del", "del", "del")])
-@pytest.mark.parametrize("m,k,n", [(512, 384, 448), (384, 512, 200), (100, 448, 384), (448, 200, 640)])
+@pytest.mark.parametrize("m,k,n", [(512, 384, 448), (384, 512, 200), (100, 448, 384), (448, 200, 640),
+                                   (512, 384, 640), (384, 768, 512), (1152, 640, 384)])
 def test_fused_path_with_k_blocked_operands_equals_the_composed_pipeline(f8, scaling, m, k, n):
     """Sizes at which some or all of the three GEMMs take k-blocked operands (contraction a multiple
-    of 64 and >= 384) against the composed, row-major pipeline: identical bits everywhere."""
+    of 64 and >= 384), and sizes at which every tensor is cast once and read transposed by the GEMM that
+    contracts its other dimension (all three multiples of 128), against the composed, row-major
+    pipeline: identical bits everywhere."""
     torch.manual_seed(2)
     lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
     a = f8.Float8Linear.from_float(copy.deepcopy(lin), config=_cfg(f8, *scaling)).to(DEV)
@@ -224,6 +227,27 @@ def test_fused_path_with_k_blocked_operands_equals_the_composed_pipeline(f8, sca
             outs.append((y, xi.grad, mod.weight.grad))
         for u, v in zip(*outs):
             assert torch.equal(u, v)
+
+
+@pytest.mark.parametrize("frozen", ["weight", "input"])
+def test_single_copy_path_with_one_gradient_not_needed(f8, frozen):
+    torch.manual_seed(4)
+    m, k, n = 384, 512, 640
+    lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
+    a = f8.Float8Linear.from_float(copy.deepcopy(lin)).to(DEV)
+    b = f8.Float8Linear.from_float(copy.deepcopy(lin)).to(DEV)
+    x = torch.randn(m, k).to(torch.bfloat16).to(DEV)
+    dy = torch.randn(m, n).to(torch.bfloat16).to(DEV)
+    outs = []
+    for mod, fwd in ((a, a.forward), (b, b.forward_composed)):
+        mod.weight.requires_grad_(frozen != "weight")
+        xi = x.clone().requires_grad_(frozen != "input")
+        y = fwd(xi)
+        y.backward(dy)
+        outs.append((y, xi.grad, mod.weight.grad))
+    for u, v in zip(*outs):
+        assert (u is None and v is None) or torch.equal(u, v)
+    assert outs[0][1 if frozen == "input" else 2] is None
 
 
 # --------------------------------------------------------------- config 1
