@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this script, each scaled by the same counter's reading for a
 # 1 GiB device copy (x2.0 and x1.0); the summary is profiles/bench_llama70b_gemm_hbm_traffic_pmc.txt.
 # Only meaningful at the default --m.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 5.65e9
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 5.66e9
 
 
 def parse():
@@ -204,7 +204,7 @@ def main():
             "flop_convention": "3 * 2*M*K*N per shape",
         },
         "roofline": {
-            "kernel": "f8mi gemm_nt_dma16_kernel (fp8 MFMA GEMM on k-blocked operands, all 12 launches of a step)",
+            "kernel": "f8mi gemm_nt_dma16_kernel (fp8 MFMA GEMM on k-blocked operands, read as they lie or transposed; all 12 launches of a step)",
             "bound": "mfma",
             "achieved": gemm_tflops,
             "peak": PEAK_FP8_TFLOPS,
