@@ -1,0 +1,105 @@
+"""Float8Linear forward + backward captured in a HIP graph and replayed.
+
+The library allocates nothing, never synchronises and launches only kernels on the stream it is given,
+so a whole training step can be recorded once and replayed (the launch-bound regime of small layers).
+Every replay is checked bit for bit against the eager result on the same inputs, with eager work and
+synchronisation between the replays.
+"""
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def f8():
+    if not torch.cuda.is_available():
+        pytest.fail("these tests need a GPU (run with -m gpu on an MI355X box)")
+    import float8_experimental_amd as pkg
+    from float8_experimental_amd import _native
+
+    _native.lib()
+    return pkg
+
+
+def _capture(fn, warmup=3):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(warmup):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fn()
+    return graph, out
+
+
+@pytest.mark.parametrize("m,k,h,n", [(130, 200, 448, 96),      # row-major and mixed operand layouts
+                                     (384, 512, 640, 384)])    # one fp8 copy per tensor, read transposed
+def test_dynamic_scaling_step_replays_bitwise(f8, m, k, h, n):
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(k, h, bias=True), nn.GELU(), nn.Linear(h, n, bias=False)).to(DEV, dtype=torch.bfloat16)
+    f8.convert_to_float8_training(model)
+    params = list(model.parameters())
+    x_s = torch.randn(m, k, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    dy_s = torch.randn(m, n, device=DEV, dtype=torch.bfloat16)
+
+    def step():
+        y = model(x_s)
+        return (y,) + torch.autograd.grad(y, [x_s] + params, dy_s)
+
+    graph, outs = _capture(step)
+    for it in range(4):
+        x = torch.randn(m, k, device=DEV, dtype=torch.bfloat16) * (it + 1)
+        dy = torch.randn(m, n, device=DEV, dtype=torch.bfloat16) * 10.0 ** (it - 2)
+        with torch.no_grad():
+            x_s.copy_(x)
+            dy_s.copy_(dy)
+        graph.replay()
+        got = [o.clone() for o in outs]
+        torch.cuda.synchronize()
+        want = step()  # eager, same static inputs
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), it
+
+
+def test_delayed_scaling_step_with_sync_replays_bitwise(f8):
+    torch.manual_seed(1)
+    m, k, h, n = 256, 384, 512, 128
+    D = f8.ScalingType.DELAYED
+    cfg = f8.Float8LinearConfig(cast_config_input=f8.CastConfig(D), cast_config_weight=f8.CastConfig(D),
+                                cast_config_grad_output=f8.CastConfig(D))
+    model = nn.Sequential(nn.Linear(k, h, bias=False), nn.ReLU(), nn.Linear(h, n, bias=False)).to(DEV, dtype=torch.bfloat16)
+    f8.convert_to_float8_training(model, config=cfg)
+    params = list(model.parameters())
+    x_s = torch.randn(m, k, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    dy_s = torch.randn(m, n, device=DEV, dtype=torch.bfloat16)
+
+    def step(mod=model, ps=params):
+        f8.sync_float8_amax_and_scale_history(mod)
+        y = mod(x_s)
+        return (y,) + torch.autograd.grad(y, [x_s] + ps, dy_s)
+
+    graph, outs = _capture(step)  # the warm-up iterations initialise the amax buffers
+    twin = copy.deepcopy(model)   # same buffers as the captured model has now; stepped eagerly beside it
+    twin_params = list(twin.parameters())
+    for it in range(4):
+        with torch.no_grad():
+            x_s.copy_(torch.randn(m, k, device=DEV, dtype=torch.bfloat16) * 1.5 ** it)
+            dy_s.copy_(torch.randn(m, n, device=DEV, dtype=torch.bfloat16))
+        graph.replay()
+        got = [o.clone() for o in outs]
+        torch.cuda.synchronize()
+        want = step(twin, twin_params)
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), it
+        for (name, b1), (_, b2) in zip(model.named_buffers(), twin.named_buffers()):
+            assert torch.equal(b1, b2), (it, name)
