@@ -29,6 +29,8 @@ EXPORTS = (
     "f8mi_device_info",
     "f8mi_workspace_bytes",
     "f8mi_amax_scale",
+    "f8mi_amax_scale_multi",
+    "f8mi_amax_tile_elems",
     "f8mi_cast",
     "f8mi_cast_layout",
     "f8mi_gemm_nt",
@@ -75,6 +77,10 @@ def lib() -> C.CDLL:
         L.f8mi_workspace_bytes.argtypes = []
         L.f8mi_amax_scale.restype = i32
         L.f8mi_amax_scale.argtypes = [vp, i64, i64, i64, i32, i32, i32, i32, fp, fp, vp, vp]
+        L.f8mi_amax_scale_multi.restype = i32
+        L.f8mi_amax_scale_multi.argtypes = [vp, i32, i64, i32, i32, i32, i32, fp, fp, vp, vp]
+        L.f8mi_amax_tile_elems.restype = i64
+        L.f8mi_amax_tile_elems.argtypes = [i32]
         L.f8mi_cast.restype = i32
         L.f8mi_cast.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, vp, fp, vp, vp]
         L.f8mi_cast_layout.restype = i32
@@ -178,6 +184,52 @@ def amax_scale(x: torch.Tensor, float8_dtype: torch.dtype, math_dtype: Optional[
                                scale.data_ptr() if scale is not None else None, ws.data_ptr(), _stream(x))
     _check(rc, "f8mi_amax_scale")
     return amax, scale
+
+
+_multi_tables = {}
+
+
+def amax_scale_multi(tensors, float8_dtype: torch.dtype, math_dtype: Optional[torch.dtype] = None,
+                     orig_is_fp16: Optional[bool] = None):
+    """(amaxes [n] fp32, scales [n] fp32) of n dense tensors of one dtype on one device, in three launches
+    whatever n is.  See f8mi_amax_scale_multi.  The device table of (pointer, numel, first tile) rows is kept
+    for as long as the same tensors (same storage, same sizes) are passed again."""
+    tensors = list(tensors)
+    assert tensors, "no tensors"
+    x0 = tensors[0]
+    for t in tensors:
+        _require_gpu(t, "tensor")
+        assert t.dtype == x0.dtype and t.device == x0.device, "tensors must share dtype and device"
+        assert t.is_contiguous() and t.data_ptr() % 16 == 0, "tensors must be dense and 16-byte aligned"
+    if math_dtype is None:
+        math_dtype = x0.dtype
+    if orig_is_fp16 is None:
+        orig_is_fp16 = x0.dtype == torch.float16
+    L = lib()
+    limit = L.f8mi_workspace_bytes() // 4
+    tile = L.f8mi_amax_tile_elems(_DT[x0.dtype])
+    amaxes = torch.empty(len(tensors), dtype=torch.float32, device=x0.device)
+    scales = torch.empty(len(tensors), dtype=torch.float32, device=x0.device)
+    ws = workspace(x0.device)
+    for lo in range(0, len(tensors), limit):
+        part = tensors[lo:lo + limit]
+        key = (x0.device.index, x0.dtype) + tuple((t.data_ptr(), t.numel()) for t in part)
+        hit = _multi_tables.get(key)
+        if hit is None:
+            rows, first = [], 0
+            for t in part:
+                rows.append([t.data_ptr(), t.numel(), first])
+                first += t.numel() // tile + 1
+            if len(_multi_tables) > 64:
+                _multi_tables.clear()
+            hit = (torch.tensor(rows, dtype=torch.int64, device="cpu").to(x0.device), first)
+            _multi_tables[key] = hit
+        table, total_tiles = hit
+        rc = L.f8mi_amax_scale_multi(table.data_ptr(), len(part), total_tiles, _DT[x0.dtype], _F8[float8_dtype],
+                                     _DT[math_dtype], int(orig_is_fp16), amaxes[lo:].data_ptr(), scales[lo:].data_ptr(),
+                                     ws.data_ptr(), _stream(x0))
+        _check(rc, "f8mi_amax_scale_multi")
+    return amaxes, scales
 
 
 KB = 64          # depth of one block of the k-blocked operand layout

@@ -130,6 +130,79 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_strided_kernel(const void* 
     if (threadIdx.x == 0) ws[blockIdx.x] = m;
 }
 
+// ---- several tensors in one pass ------------------------------------------------------------
+// The tensors are cut into the same 32 KB tiles as above and the tiles numbered through all tensors
+// (entry t owns tiles [first_tile[t], first_tile[t+1]), numel / tile elements + 1 of them).  Every read is
+// guarded by the entry's own numel, whatever the tile numbers say.  A block takes a contiguous
+// range of tile numbers, so it changes tensor rarely; on every change, and at its end, it folds its
+// maximum into that tensor's workspace word with one atomic (a few per block, spread over n addresses).
+__global__ void amax_multi_zero_kernel(uint32_t* ws, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) ws[i] = 0u;
+}
+
+template <int DT>
+__global__ __launch_bounds__(AMAX_THREADS) void amax_multi_kernel(const f8mi_tensor_ref* __restrict__ refs, int n,
+                                                                   int64_t total_tiles, uint32_t* __restrict__ ws) {
+    __shared__ uint32_t red[AMAX_THREADS / 64];
+    constexpr int EPV = DT == F8MI_FP32 ? 4 : 8;
+    constexpr int64_t TILE = (int64_t)AMAX_THREADS * AMAX_UNROLL;
+    const int64_t t0 = total_tiles * blockIdx.x / gridDim.x, t1 = total_tiles * (blockIdx.x + 1) / gridDim.x;
+    if (t0 >= t1) return;
+    // the tensor that owns tile t0: last entry with first_tile <= t0
+    int lo = 0, hi = n - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (refs[mid].first_tile <= t0) lo = mid; else hi = mid - 1;
+    }
+    int cur = lo;
+    uint32_t m = 0;
+    for (int64_t t = t0; t < t1; t++) {
+        while (cur + 1 < n && refs[cur + 1].first_tile <= t) {  // block-uniform: flush and move on
+            m = block_max_u32(m, red);
+            if (threadIdx.x == 0 && m) atomicMax(&ws[cur], m);
+            __syncthreads();
+            m = 0;
+            cur++;
+        }
+        const f8mi_tensor_ref r = refs[cur];
+        const int64_t nvec = r.numel / EPV;
+        const uint4* xv = (const uint4*)r.data;
+        const int64_t base = (t - r.first_tile) * TILE + threadIdx.x;
+        uint4 v[AMAX_UNROLL];
+        if (base - threadIdx.x + TILE <= nvec) {
+#pragma unroll
+            for (int u = 0; u < AMAX_UNROLL; u++) v[u] = load_nt16(&xv[base + u * AMAX_THREADS]);
+        } else {
+#pragma unroll
+            for (int u = 0; u < AMAX_UNROLL; u++) {
+                const int64_t i = base + u * AMAX_THREADS;
+                v[u] = i < nvec ? load_nt16(&xv[i]) : make_uint4(0, 0, 0, 0);
+            }
+            // numel / (elements per tile) + 1 tiles per tensor: the last one is always partial (possibly without
+            // any whole vector) and also takes the < EPV trailing elements
+            const int64_t e = nvec * EPV + threadIdx.x;
+            if (e < r.numel && base - threadIdx.x + TILE > nvec && base - threadIdx.x <= nvec) {
+                const uint32_t a = absmax_elem<DT>(r.data, e);
+                m = m > a ? m : a;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < AMAX_UNROLL; u++) m = absmax_vec<DT>(v[u], m);
+    }
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0 && m) atomicMax(&ws[cur], m);
+}
+
+__global__ void amax_multi_finalize_kernel(const uint32_t* __restrict__ ws, int n, float* amax_out, float* scale_out,
+                                           int in_dt, int math_dt, int fmt, int orig_is_fp16) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float amax = abs_bits_to_float(ws[i], in_dt);
+    if (amax_out) amax_out[i] = amax;
+    if (scale_out) scale_out[i] = amax_to_scale_dev(amax, math_dt, fmt, orig_is_fp16);
+}
+
 // Empty tensor: torch.max raises; we define amax = 0 so the scale is fmax/eps.
 __global__ void amax_empty_kernel(float* amax_out, float* scale_out, int math_dt, int fmt, int orig_is_fp16) {
     if (threadIdx.x == 0) {
@@ -201,4 +274,36 @@ extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_
     hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(AMAX_THREADS), 0, stream, ws, (int)blocks, amax_dev, scale_dev, in_dtype,
                        math_dtype, fp8_fmt, orig_is_fp16);
     return check_hip(hipGetLastError(), "amax finalize kernel launch");
+}
+
+extern "C" int f8mi_amax_scale_multi(const f8mi_tensor_ref* refs_dev, int n, int64_t total_tiles, int in_dtype, int fp8_fmt,
+                                     int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
+                                     void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n < 0 || n > WS_WORDS) { set_error("f8mi_amax_scale_multi: n=%d tensors, at most %d per call", n, WS_WORDS); return F8MI_ERR_INVALID_ARG; }
+    if (in_dtype < 0 || in_dtype > 2 || math_dtype < 0 || math_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_amax_scale_multi: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
+    if (!amax_dev && !scale_dev) { set_error("f8mi_amax_scale_multi: no output requested"); return F8MI_ERR_INVALID_ARG; }
+    if (n == 0) return F8MI_OK;
+    if (!refs_dev || !workspace || total_tiles < n) { set_error("f8mi_amax_scale_multi: null table or workspace, or fewer tiles than tensors"); return F8MI_ERR_INVALID_ARG; }
+    uint32_t* ws = (uint32_t*)workspace;
+    hipLaunchKernelGGL(amax_multi_zero_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, ws, n);
+    int64_t blocks = (int64_t)cu_count() * 2;
+    if (blocks > total_tiles) blocks = total_tiles;
+    {
+        // profiling counter: tiles * 32 KB, an upper bound of the bytes read (less than one tile per tensor too many)
+        ProfScope prof(F8MI_K_AMAX, (double)total_tiles * AMAX_THREADS * AMAX_UNROLL * 16, stream);
+        dim3 g((unsigned)blocks), b(AMAX_THREADS);
+        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_multi_kernel<F8MI_BF16>, g, b, 0, stream, refs_dev, n, total_tiles, ws);
+        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_multi_kernel<F8MI_FP16>, g, b, 0, stream, refs_dev, n, total_tiles, ws);
+        else hipLaunchKernelGGL(amax_multi_kernel<F8MI_FP32>, g, b, 0, stream, refs_dev, n, total_tiles, ws);
+    }
+    int rc = check_hip(hipGetLastError(), "amax multi kernel launch");
+    if (rc) return rc;
+    hipLaunchKernelGGL(amax_multi_finalize_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, ws, n, amax_dev, scale_dev, in_dtype,
+                       math_dtype, fp8_fmt, orig_is_fp16);
+    return check_hip(hipGetLastError(), "amax multi finalize kernel launch");
+}
+
+extern "C" int64_t f8mi_amax_tile_elems(int in_dtype) {
+    return (int64_t)AMAX_THREADS * AMAX_UNROLL * (in_dtype == F8MI_FP32 ? 4 : 8);
 }

@@ -4,9 +4,10 @@
 The reference strings the layer together from four autograd functions and a tensor
 subclass (cast x, cast W, matmul, cast dY in backward).  Here the whole layer is ONE
 autograd function around five kernel launches per direction: amax+scale and
-cast(+transposed copy) per tensor, and one matrix-core GEMM per product.  The
-transposed fp8 copies the backward GEMMs need are written by the cast kernels while
-the data is in registers, and only those transposed copies are kept for backward.
+cast per tensor, and one matrix-core GEMM per product.  Where the sizes allow it each
+tensor has ONE fp8 copy and the backward GEMMs read it transposed; otherwise the
+transposed fp8 copies are written by the cast kernels while the data is in registers,
+and only those are kept for backward.
 The pieces of the reference's composition (``cast_input_to_float8`` ...,
 ``manual_float8_matmul``) are still here and give the same numbers.
 """
@@ -24,7 +25,13 @@ from .float8_scaling_utils import (
     NoopFwToFloat8E5M2BwDelayed,
     NoopFwToFloat8E5M2BwDynamic,
 )
-from .float8_tensor import Float8Tensor, GemmInputRole, LinearMMConfig, ScaledMMConfig
+from .float8_tensor import (
+    Float8Tensor,
+    GemmInputRole,
+    LinearMMConfig,
+    ScaledMMConfig,
+    hp_tensor_and_scale_to_float8,
+)
 from .float8_utils import e4m3_dtype, e5m2_dtype
 
 _KINDS = ("input", "weight", "grad_output")
@@ -62,7 +69,8 @@ class _DelayedBuffers:
 
 
 def _cast_for_gemm(t2d: torch.Tensor, float8_dtype, delayed: Optional[_DelayedBuffers], is_initialized: bool,
-                   want_row: bool, want_t: bool, row_kb: bool = False, t_kb: bool = False):
+                   want_row: bool, want_t: bool, row_kb: bool = False, t_kb: bool = False,
+                   known_scale: Optional[torch.Tensor] = None):
     """fp8 copies of a 2-D tensor for the GEMMs: (as is, transposed, scale).
 
     dynamic: one amax+scale launch, one cast launch (float8_utils.py:115-120 +
@@ -70,9 +78,14 @@ def _cast_for_gemm(t2d: torch.Tensor, float8_dtype, delayed: Optional[_DelayedBu
     then ONE launch that casts with the existing scale and records this step's amax
     (float8_scaling_utils.py:65-125).  ``row_kb`` / ``t_kb`` ask for the k-blocked layout
     of the respective copy (same bytes, placed [k/64][rows][64] for the GEMM that contracts it).
+    ``known_scale`` (dynamic scaling only): a scale computed beforehand for exactly this tensor
+    (``precompute_float8_dynamic_scale_for_fsdp``); the amax pass is skipped.
     """
     if delayed is None:
-        _, scale = _native.amax_scale(t2d, float8_dtype, want_amax=False)
+        if known_scale is not None:
+            scale = known_scale
+        else:
+            _, scale = _native.amax_scale(t2d, float8_dtype, want_amax=False)
         row, tr = _native.cast(t2d, scale, float8_dtype, product_dtype=t2d.dtype, want_out=want_row, want_out_t=want_t,
                                out_kblock=row_kb, out_t_kblock=t_kb)
         return row, tr, scale
@@ -111,7 +124,8 @@ class _float8_linear_fn(torch.autograd.Function):
         tn = not emulate and not emulate_bw and _native.tn_ok(m, k, n)
         if tn:
             x8, _, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, False, True, False)
-            w8, _, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, False, True, False)
+            w8, _, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, False, True, False,
+                                        known_scale=mod._precomputed_weight_scale)
             y = _native.gemm_nt_kb(x8, sx, w8, sw, x.dtype)
             ctx.kb = None
             ctx.save_for_backward(x8, w8, sx, sw)
@@ -120,7 +134,8 @@ class _float8_linear_fn(torch.autograd.Function):
             kb_dx = not emulate_bw and _native.kblock_ok(n)    # dx = dy W contracts out_features
             kb_dw = not emulate_bw and _native.kblock_ok(m)    # dw = dy^T x contracts tokens
             x8, x8t, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, need_dw, kb_fwd, kb_dw)
-            w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx, kb_fwd, kb_dx)
+            w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx, kb_fwd, kb_dx,
+                                          known_scale=mod._precomputed_weight_scale)
             if emulate:
                 y = mm_float8_emulated(x8, sx, w8.t(), sw, x.dtype)
             else:
@@ -175,8 +190,12 @@ class Float8Linear(torch.nn.Linear):
         config = kwargs.pop("config")
         super().__init__(*args, **kwargs)
         self.config = config
-        if config.enable_fsdp_float8_all_gather:
-            raise NotImplementedError("enable_fsdp_float8_all_gather needs FSDP2 over several GPUs; this build drives one GPU")
+        # enable_fsdp_float8_all_gather: the one-GPU share of that flow is kept -- the weight's scale may be
+        # computed ahead of the forward pass, for all layers in one launch
+        # (precompute_float8_dynamic_scale_for_fsdp), and the forward then casts the weight with it.  The
+        # reference wraps the weight in a tensor subclass for FSDP2's all-gather hooks; with one GPU there is
+        # nothing to gather and the parameter stays a plain tensor.
+        self._precomputed_weight_scale = None
 
         self.scaling_type_input = config.cast_config_input.scaling_type
         self.scaling_type_weight = config.cast_config_weight.scaling_type
@@ -260,6 +279,9 @@ class Float8Linear(torch.nn.Linear):
                                                linear_mm_config=self.linear_mm_config,
                                                gemm_input_role=GemmInputRole.WEIGHT)
         assert self.scaling_type_weight is ScalingType.DYNAMIC
+        if self._precomputed_weight_scale is not None:  # what fsdp_pre_all_gather does (fsdp_utils.py:166-174)
+            return hp_tensor_and_scale_to_float8(self.weight, self._precomputed_weight_scale, e4m3_dtype,
+                                                 self.linear_mm_config, GemmInputRole.WEIGHT)
         return hp_tensor_to_float8_dynamic(self.weight, e4m3_dtype, self.linear_mm_config,
                                            gemm_input_role=GemmInputRole.WEIGHT)
 
@@ -311,7 +333,7 @@ class Float8Linear(torch.nn.Linear):
     def _forward_under_compile(self, input: torch.Tensor) -> torch.Tensor:
         """What ``torch.compile`` traces: all-dynamic scaling is one custom-op node (plus the bias add);
         anything that keeps state on the module, or carries Float8Tensors, runs outside the graph."""
-        plain = (not self.has_any_delayed_scaling and not self.config.emulate
+        plain = (not self.has_any_delayed_scaling and not self.config.emulate and self._precomputed_weight_scale is None
                  and not isinstance(self.weight, Float8Tensor) and not isinstance(input, Float8Tensor))
         if not plain:
             return self._forward_outside_graph(input)

@@ -80,6 +80,30 @@ int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_t ld, int i
                     int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
                     void* stream);
 
+/* One tensor of a list given to f8mi_amax_scale_multi. */
+typedef struct f8mi_tensor_ref {
+    const void* data;   /* dense, 16-byte aligned, `numel` elements of the call's in_dtype */
+    int64_t numel;
+    int64_t first_tile; /* number of tiles of all entries before this one; an entry has
+                           numel / f8mi_amax_tile_elems(in_dtype) + 1 tiles */
+} f8mi_tensor_ref;
+
+/* Elements of `in_dtype` in one tile (32 KB) of f8mi_amax_scale_multi's numbering. */
+int64_t f8mi_amax_tile_elems(int in_dtype);
+
+/*
+ * amax and scale of n tensors in one pass: amax_dev[i], scale_dev[i] (either may be NULL) as
+ * f8mi_amax_scale gives them for tensor i.  Replaces the torch._foreach_norm(weights, ord=inf)
+ * + stack + clamp + divide chain of precompute_float8_dynamic_scale_for_fsdp
+ * (fsdp_utils.py:59-66) -- the per-GPU part of it; the all-reduce between ranks is the caller's.
+ *   refs_dev     device array of n entries (n <= f8mi_workspace_bytes() / 4)
+ *   total_tiles  sum of the entries' tile counts
+ * Three launches whatever n is.
+ */
+int f8mi_amax_scale_multi(const f8mi_tensor_ref* refs_dev, int n, int64_t total_tiles, int in_dtype, int fp8_fmt,
+                          int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
+                          void* stream);
+
 /*
  * Saturated cast to fp8: bytes = fp8(clamp(x * scale, -fmax, fmax)), round to
  * nearest even.  Replaces _ToFloat8ConstrFunc.forward (float8_tensor.py:139-191)

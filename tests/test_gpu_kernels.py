@@ -91,6 +91,49 @@ def test_amax_specials(nat):
     assert a.item() == 0.5
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+def test_amax_of_many_tensors_in_one_pass_matches_oracle(nat, dt):
+    """f8mi_amax_scale_multi: sizes around the tile (32 KB) and vector (16 B) boundaries, an empty tensor,
+    a NaN and an inf, against the oracle and against the one-tensor entry point, bit for bit."""
+    co, to = _oracles()
+    tdt = TORCH_DT[dt]
+    tile = nat.lib().f8mi_amax_tile_elems(nat._DT[tdt])
+    sizes = [1, 7, 8, 9, 0, tile - 1, tile, tile + 1, 3 * tile, 3 * tile + 5, 1000003, 5 * tile - 8, 2, 20 * tile + 3]
+    hosts = [heavy((n,), tdt, 10 + i) * (0.01 * (i + 1)) for i, n in enumerate(sizes)]
+    hosts[5][-1] = float("nan")          # in the partial last tile
+    hosts[8][tile + 17] = float("-inf")  # in a whole tile
+    hosts[9][-1] = 3.0e4                 # the maximum sits in the < 16-byte tail
+    devs = [h.to(DEV) for h in hosts]
+    for fmt, (code, f8dt) in F8.items():
+        amaxes, scales = nat.amax_scale_multi(devs, f8dt)
+        assert amaxes.shape == scales.shape == (len(sizes),)
+        for i, (h, d) in enumerate(zip(hosts, devs)):
+            a1, s1 = nat.amax_scale(d, f8dt)
+            assert amaxes[i].view(torch.int32).item() == a1.view(torch.int32).item(), (dt, fmt, sizes[i])
+            assert scales[i].view(torch.int32).item() == s1.view(torch.int32).item(), (dt, fmt, sizes[i])
+            if h.numel() and not torch.isnan(h).any():
+                assert amaxes[i].item() == to.tensor_to_amax(h).float().item()
+                assert scales[i].cpu().view(torch.int32).item() == to.tensor_to_scale(h, f8dt).view(torch.int32).item()
+        assert torch.isnan(amaxes[5]).item() and torch.isnan(scales[5]).item()
+        assert amaxes[8].item() == float("inf") and scales[8].item() == 0.0
+    # the same list again (cached table) after the data changed
+    devs[0].fill_(5.0)
+    amaxes, _ = nat.amax_scale_multi(devs, torch.float8_e4m3fn)
+    assert amaxes[0].item() == 5.0
+
+
+def test_amax_of_more_tensors_than_one_call_takes(nat):
+    n = nat.lib().f8mi_workspace_bytes() // 4 + 300
+    torch.manual_seed(5)
+    big = torch.randn(n, 24, device=DEV).to(torch.bfloat16)  # rows of 48 bytes: 16-byte aligned
+    rows = [big[i] for i in range(n)]
+    amaxes, scales = nat.amax_scale_multi(rows, torch.float8_e5m2)
+    want = big.abs().amax(dim=1).float()
+    assert torch.equal(amaxes, want)
+    _, s = nat.amax_scale(rows[n - 1], torch.float8_e5m2)
+    assert scales[n - 1].item() == s.item()
+
+
 @pytest.mark.parametrize("dt", ["bf16", "fp16"])
 def test_scale_math_sweep_16bit(nat, dt):
     """Scale arithmetic in the tensor's own dtype over a sweep of amax bit patterns."""

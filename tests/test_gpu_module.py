@@ -250,6 +250,46 @@ def test_single_copy_path_with_one_gradient_not_needed(f8, frozen):
     assert outs[0][1 if frozen == "input" else 2] is None
 
 
+# --------------------------------------------------------------- scales computed ahead of the forward
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+def test_precomputed_weight_scales_give_the_same_step(f8, dt):
+    """precompute_float8_dynamic_scale_for_fsdp on one GPU: all weight scales in one pass; the forward that
+    uses them equals the forward that computes each scale itself, fused and composed, bit for bit."""
+    from float8_experimental_amd import _native
+
+    torch.manual_seed(6)
+    dims = [(384, 512), (512, 200), (200, 384)]
+    base = nn.Sequential(*[nn.Linear(k, n, bias=(i == 1)) for i, (k, n) in enumerate(dims)]).to(dt)
+    cfg = f8.Float8LinearConfig(enable_fsdp_float8_all_gather=True)
+    a = f8.convert_to_float8_training(copy.deepcopy(base), config=cfg).to(DEV)
+    b = f8.convert_to_float8_training(copy.deepcopy(base)).to(DEV)
+    opt_a = torch.optim.SGD(a.parameters(), lr=0.1)
+    opt_b = torch.optim.SGD(b.parameters(), lr=0.1)
+    for it in range(3):
+        x = torch.randn(384, 384).to(dt).to(DEV)
+        dy = torch.randn(384, 384).to(dt).to(DEV)
+        f8.precompute_float8_dynamic_scale_for_fsdp(a)
+        for lay_a, lay_b in zip(a, b):
+            _, s = _native.amax_scale(lay_b.weight.detach(), torch.float8_e4m3fn)
+            assert lay_a._precomputed_weight_scale.item() == s.item()
+        outs = []
+        for mod, opt, composed in ((a, opt_a, it == 2), (b, opt_b, False)):
+            opt.zero_grad(set_to_none=True)
+            xi = x.clone().requires_grad_()
+            h = xi
+            for lay in mod:
+                h = lay.forward_composed(h) if composed else lay(h)
+            h.backward(dy)
+            outs.append([h.detach(), xi.grad] + [p.grad.clone() for p in mod.parameters()])
+            opt.step()
+        for u, v in zip(*outs):
+            assert torch.equal(u, v), it
+    assert f8.precompute_float8_dynamic_scale_for_fsdp(b) is None  # no layer of b carries the flag
+    assert all(lay._precomputed_weight_scale is None for lay in b)
+
+
 # --------------------------------------------------------------- config 1
 
 

@@ -186,11 +186,22 @@ def test_sync_host_checks(caplog):
         sync_float8_amax_and_scale_history(mixed)
 
 
-def test_fsdp_and_multi_gpu_entry_points_say_so():
+def test_fsdp_flag_and_precompute_on_the_host():
+    """enable_fsdp_float8_all_gather keeps its one-GPU meaning (scales of all weights computed ahead, in one pass);
+    the host-side rules follow the reference (fsdp_utils.py:29-66)."""
+    from float8_experimental_amd._native import Float8NativeError
+
+    lin = Float8Linear.from_float(nn.Linear(4, 4), config=Float8LinearConfig(enable_fsdp_float8_all_gather=True))
+    assert lin._precomputed_weight_scale is None
+    # nothing to do: no layer was created with the flag (the reference returns silently as well)
+    assert f8.precompute_float8_dynamic_scale_for_fsdp(nn.Linear(4, 4)) is None
+    assert f8.precompute_float8_dynamic_scale_for_fsdp(nn.Sequential(Float8Linear.from_float(nn.Linear(4, 4)))) is None
+    # delayed weight scaling anywhere in the model is refused
     with pytest.raises(NotImplementedError):
-        Float8Linear.from_float(nn.Linear(4, 4), config=Float8LinearConfig(enable_fsdp_float8_all_gather=True))
-    with pytest.raises(NotImplementedError):
-        f8.precompute_float8_dynamic_scale_for_fsdp(nn.Linear(4, 4))
+        f8.precompute_float8_dynamic_scale_for_fsdp(nn.Sequential(Float8Linear.from_float(nn.Linear(4, 4), config=cfg(DYN, DEL, DYN))))
+    # and the computation itself needs the GPU: no CPU fallback
+    with pytest.raises(Float8NativeError):
+        f8.precompute_float8_dynamic_scale_for_fsdp(nn.Sequential(lin))
 
 
 def test_float8_tensor_metadata_on_cpu():
