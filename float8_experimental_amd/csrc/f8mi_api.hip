@@ -44,14 +44,14 @@ ProfScope::ProfScope(int kernel_, double work_, hipStream_t stream_) : kernel(ke
     if (!g_prof_on) return;
     ProfRec* r = new ProfRec{kernel, work, nullptr, nullptr};
     if (hipEventCreate(&r->start) != hipSuccess || hipEventCreate(&r->stop) != hipSuccess) { delete r; return; }
-    hipEventRecord(r->start, stream);
+    (void)hipEventRecord(r->start, stream);
     rec = r;
 }
 
 ProfScope::~ProfScope() {
     if (!rec) return;
     ProfRec* r = (ProfRec*)rec;
-    hipEventRecord(r->stop, stream);
+    (void)hipEventRecord(r->stop, stream);
     std::lock_guard<std::mutex> lk(g_prof_mu);
     g_prof_recs.push_back(r);
 }
@@ -64,8 +64,8 @@ static void prof_drain_locked() {
             g_prof_ms[r->kernel] += ms;
             g_prof_work[r->kernel] += r->work;
         }
-        hipEventDestroy(r->start);
-        hipEventDestroy(r->stop);
+        (void)hipEventDestroy(r->start);
+        (void)hipEventDestroy(r->stop);
         delete r;
     }
     g_prof_recs.clear();

@@ -162,6 +162,11 @@ static int allow_big_lds(K kern, int bytes, std::atomic<uint64_t>& done_mask) {
 
 // The 16x16x128 kernel with Bt (nt) or both operands (tt) given transposed: memory holds [contraction][rows];
 // lda / ldb = bytes between contraction rows, a_unit / b_unit = bytes between blocks of 64 rows.
+// few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands
+constexpr int SKINNY_MAX_M = 128;
+int launch_gemm_skinny(int a_fmt, int b_fmt, int c_dtype, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
+                       const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
+                       int64_t ldc, const void* bias);
 int launch_gemm_dma16_nt(int a_fmt, int b_fmt, int c_dtype, dim3 g, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                          const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb,
                          void* C, int64_t ldc, const void* bias, int tiles_m, int tiles_n, int c_vec_ok);

@@ -369,6 +369,31 @@ def test_gemm_dma_kernel_shapes(nat, m, n, k, out_dt):
     _gemm_check(nat, m, n, k, "e5m2", "e4m3", out_dt, seed=m + n + k, bias=(m % 2 == 0))
 
 
+# Few rows (m <= 128, k % 128 == 0, aligned): the kernel that streams Bt straight into the matrix cores and splits k
+# over the eight waves of a workgroup.  m around the 16-row tile edges, n ragged against the 32-column
+# workgroups, k from one step (seven idle waves) over nine (uneven split) to a long one.
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 33, 64, 65, 100, 128])
+@pytest.mark.parametrize("n,k", [(7, 128), (32, 256), (200, 1152), (1000, 1024), (96, 8192)])
+def test_gemm_few_rows_shapes(nat, m, n, k):
+    fm = [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2"), ("e5m2", "e5m2")][(m + n) % 4]
+    out_dt = [torch.bfloat16, torch.float32, torch.float16][(m + k // 128) % 3]
+    _gemm_check(nat, m, n, k, fm[0], fm[1], out_dt, seed=m + n + k, bias=(m % 2 == 1))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (16, 520, 2048), (48, 1000, 640), (64, 264, 8192), (120, 264, 1024)])
+def test_gemm_few_rows_kblocked_equals_row_major_bitwise(nat, m, n, k):
+    a = _rand_fp8((m, k), torch.float8_e4m3fn, m + k, 4.0).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e4m3fn, n + k, 4.0).to(DEV)
+    sa, sb = torch.tensor(2.0, device=DEV), torch.tensor(0.25, device=DEV)
+    bias = torch.randn(n, device=DEV).to(torch.bfloat16)
+    want = nat.gemm_nt(a, sa, bt, sb, torch.bfloat16, bias=bias)
+    got = nat.gemm_nt_kb(_to_kb(a), sa, _to_kb(bt), sb, torch.bfloat16, bias=bias)
+    assert torch.equal(got, want)
+    # rows are independent: any subset of A's rows gives the same rows of C, whichever tile count it lands in
+    sub = nat.gemm_nt(a[: max(1, m // 3)].contiguous(), sa, bt, sb, torch.bfloat16, bias=bias)
+    assert torch.equal(sub, want[: max(1, m // 3)])
+
+
 def test_gemm_kernels_agree_bitwise(nat):
     """Same operands through the LDS-DMA kernel (aligned view) and the register-staged kernel (the same
     values at a 1-byte offset, which forces the unaligned path): identical accumulation order, identical bits."""
