@@ -591,6 +591,45 @@ def test_full_size_properties_llama70b_wo(nat):
     torch.testing.assert_close(g[:, :512], g[:, :512].t(), rtol=1e-5, atol=1e-3)
 
 
+def test_tensors_of_more_than_2_31_elements(nat):
+    """Index arithmetic past 32 bits: amax, cast (all layouts) and the GEMM's output addressing on a tensor of
+    2.29e9 elements, checked on slices against torch's own ops on the GPU (the cast is the same function of
+    (x, scale) everywhere, so slices pin it) and on planted maxima."""
+    rows, cols = 70000, 32768
+    assert rows * cols > 2**31
+    g = torch.Generator(device=DEV).manual_seed(11)
+    x = torch.empty(rows, cols, device=DEV, dtype=torch.bfloat16).normal_(generator=g)
+    x[rows - 1, cols - 3] = 1000.0   # the maximum sits past element 2^31
+    amax, scale = nat.amax_scale(x, torch.float8_e4m3fn)
+    assert amax.item() == 1000.0
+    x[rows - 1, cols - 3] = 0.5
+    x[17, 5] = -2000.0
+    amax, scale = nat.amax_scale(x, torch.float8_e4m3fn)
+    assert amax.item() == 2000.0
+    ams, _ = nat.amax_scale_multi([x[:3], x], torch.float8_e4m3fn)
+    assert ams[1].item() == 2000.0
+    ref_rows = [0, 1, 127, 128, 32767, 65535, 65536, rows - 129, rows - 2, rows - 1]
+    want = (x[ref_rows] * scale).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    out, out_t = nat.cast(x, scale, torch.float8_e4m3fn, want_out_t=True)
+    assert torch.equal(out[ref_rows].view(torch.uint8), want)
+    assert torch.equal(out_t[:, ref_rows].view(torch.uint8), want.t())
+    del out_t
+    okb, _ = nat.cast(x, scale, torch.float8_e4m3fn, out_kblock=True)  # [cols/64, rows, 64]
+    assert torch.equal(okb[:, ref_rows, :].view(torch.uint8).permute(1, 0, 2).reshape(len(ref_rows), cols), want)
+    del okb
+    # GEMM with more than 2^31 outputs: C = out[:, :384] (70000 x 384) times a 32768 x 384 matrix
+    a8 = out[:, :384].contiguous()
+    b8 = _rand_fp8((cols, 384), torch.float8_e4m3fn, 3, 2.0).to(DEV)
+    one = torch.ones((), device=DEV)
+    c = nat.gemm_nt(a8, one, b8, one, torch.bfloat16)
+    assert c.numel() > 2**31
+    for r0 in (0, 65536 - 128, rows - 256):
+        ref = nat.gemm_nt(a8[r0:r0 + 256].contiguous(), one, b8, one, torch.bfloat16)
+        assert torch.equal(c[r0:r0 + 256], ref), r0
+    exact = a8[rows - 64:].double() @ b8.double().t()
+    torch.testing.assert_close(c[rows - 64:].double(), exact, rtol=2.0**-7, atol=0.5)
+
+
 def test_mfma_probe_reports_a_sane_ceiling(nat):
     """f8mi_probe_mfma: register-only MFMA loop; zeros run at the clock limit, random bytes below it."""
     zero = nat.probe_mfma(False, iters=1000)
