@@ -42,6 +42,9 @@ def parse():
     p.add_argument("--steps", type=int, default=5)
     p.add_argument("--warmup", type=int, default=2)
     p.add_argument("--m", type=int, default=M_TOKENS, help="tokens per step (default: the benchmark's 16384)")
+    p.add_argument("--scaling", choices=["dynamic", "delayed"], default="dynamic",
+                   help="dynamic (the headline configuration) or delayed scaling of all three tensors with one "
+                        "sync_float8_amax_and_scale_history per step")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-bf16", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the oracle sample")
@@ -50,18 +53,25 @@ def parse():
     return p.parse_args()
 
 
-def make_layers(torch, f8, m, device):
+def make_layers(torch, f8, m, device, scaling="dynamic"):
     layers = []
+    if scaling == "delayed":
+        cc = f8.CastConfig(f8.ScalingType.DELAYED)
+        config = f8.Float8LinearConfig(cast_config_input=cc, cast_config_weight=cc, cast_config_grad_output=cc)
+    else:
+        config = f8.Float8LinearConfig()
     for name, k, n in SHAPES:
         lin = torch.nn.Linear(k, n, bias=False, device=device, dtype=torch.bfloat16)  # kaiming-uniform init
-        mod = f8.Float8Linear.from_float(lin, config=f8.Float8LinearConfig())
+        mod = f8.Float8Linear.from_float(lin, config=config)
         x = torch.randn(m, k, device=device, dtype=torch.bfloat16).requires_grad_()
         dy = (torch.randn(m, n, device=device, dtype=torch.float32) * 1e-2).to(torch.bfloat16)
         layers.append((name, k, n, lin, mod, x, dy))
     return layers
 
 
-def step(layers, use_fp8=True):
+def step(layers, use_fp8=True, sync=None):
+    if sync is not None and use_fp8:
+        sync()
     for name, k, n, lin, mod, x, dy in layers:
         x.grad = None
         lin.weight.grad = None
@@ -128,7 +138,11 @@ def main():
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
     m = args.m
-    layers = make_layers(torch, f8, m, dev)
+    layers = make_layers(torch, f8, m, dev, args.scaling)
+    sync = None
+    if args.scaling == "delayed":
+        model = torch.nn.ModuleList([lay[4] for lay in layers])
+        sync = lambda: f8.sync_float8_amax_and_scale_history(model)
     flop_per_shape = {name: 3 * 2.0 * m * k * n for name, k, n, *_ in layers}
     flop_step = sum(flop_per_shape.values())
 
@@ -141,13 +155,13 @@ def main():
 
     # ---- the timed region: K steps, every kernel launch bracketed by HIP events on its stream
     for _ in range(args.warmup):
-        step(layers)
+        step(layers, sync=sync)
     torch.cuda.synchronize()
     _native.prof_reset()
     _native.prof_enable(True)
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step(layers)
+        step(layers, sync=sync)
     torch.cuda.synchronize()
     sec_step = (time.perf_counter() - t0) / args.steps
     _native.prof_enable(False)
@@ -168,7 +182,8 @@ def main():
     per_shape = {}
     for lay in layers:
         name = lay[0]
-        t = timed(torch, lambda: step([lay]), max(2, args.steps // 2), 1)
+        one_sync = (lambda: f8.sync_float8_amax_and_scale_history(lay[4])) if sync is not None else None
+        t = timed(torch, lambda: step([lay], sync=one_sync), max(2, args.steps // 2), 1)
         per_shape[name] = {"fp8_ms": t * 1e3, "fp8_TFLOP/s": flop_per_shape[name] / t / 1e12}
     bf16_step = None
     if not args.no_bf16:
@@ -198,7 +213,7 @@ def main():
         "dtype": "fp8",
         "data": "synthetic",
         "config": {
-            "workload": f"LLaMa-2-70B linear shapes, dynamic scaling, M={m} tokens bf16, (K->N) 8192->10240, 8192->8192, "
+            "workload": f"LLaMa-2-70B linear shapes, {args.scaling} scaling, M={m} tokens bf16, (K->N) 8192->10240, 8192->8192, "
                         "8192->57344, 28672->8192; fwd+bwd with dY ~N(0,1e-2); one step = all four shapes",
             "flop_per_step": flop_step,
             "flop_convention": "3 * 2*M*K*N per shape",

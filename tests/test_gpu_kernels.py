@@ -394,6 +394,47 @@ def test_gemm_few_rows_kblocked_equals_row_major_bitwise(nat, m, n, k):
     assert torch.equal(sub, want[: max(1, m // 3)])
 
 
+def test_gemm_random_sweep_over_all_dispatch_paths(nat):
+    """Seeded random (m, n, k), formats, output types, bias, row strides and 16-byte misalignment: whichever kernel
+    the library picks (few-row, 16x16x128 or 32x32x64 LDS-DMA, register-staged) the result is within the stated
+    tolerance of the exact product, and equal bit for bit to the same call on a dense, aligned copy when both take
+    the same kernel family."""
+    rng = np.random.default_rng(2024)
+    fmts = ["e4m3", "e5m2"]
+    outs = [torch.bfloat16, torch.float32, torch.float16]
+    one = None
+    for case in range(48):
+        kind = case % 6
+        m = int(rng.choice([1, 3, 16, 40, 64, 100, 128, 129, 255, 256, 300, 513]))
+        n = int(rng.choice([1, 8, 31, 64, 200, 256, 257, 520]))
+        k = int(rng.choice([[16, 48, 100, 129, 250], [128, 256, 1152], [384, 640, 1024, 2048], [448, 576, 704],
+                            [392, 1000, 4097], [128, 384, 512]][kind]))
+        a_fmt, b_fmt = fmts[int(rng.integers(2))], fmts[int(rng.integers(2))]
+        out_dt = outs[int(rng.integers(3))]
+        _gemm_check(nat, m, n, k, a_fmt, b_fmt, out_dt, seed=1000 + case, bias=bool(rng.integers(2)))
+        # the same product from operands with a padded row stride, and from operands shifted off 16-byte alignment
+        ta, tb = F8[a_fmt][1], F8[b_fmt][1]
+        a = _rand_fp8((m, k), ta, 2000 + case, 4.0).to(DEV)
+        bt = _rand_fp8((n, k), tb, 3000 + case, 4.0).to(DEV)
+        if one is None:
+            one = torch.ones((), device=DEV)
+        want = nat.gemm_nt(a, one, bt, one, torch.float32)
+        pad = 16 * int(rng.integers(1, 5))
+        a_p = torch.zeros(m, k + pad, dtype=torch.uint8, device=DEV).view(ta)
+        b_p = torch.zeros(n, k + pad, dtype=torch.uint8, device=DEV).view(tb)
+        a_p[:, :k].view(torch.uint8).copy_(a.view(torch.uint8))
+        b_p[:, :k].view(torch.uint8).copy_(bt.view(torch.uint8))
+        got = nat.gemm_nt(a_p[:, :k], one, b_p[:, :k], one, torch.float32)
+        if k % 16 == 0:
+            assert torch.equal(got, want), (case, m, n, k, "padded rows")  # same kernel: strides only
+        else:
+            torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-2)
+        a_o = torch.empty(m * k + 3, dtype=torch.uint8, device=DEV)[3:].view(ta).view(m, k)
+        a_o.view(torch.uint8).copy_(a.view(torch.uint8))
+        got = nat.gemm_nt(a_o, one, bt, one, torch.float32)   # unaligned: the register-staged kernel
+        torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-2 * max(1.0, k / 256))
+
+
 def test_gemm_kernels_agree_bitwise(nat):
     """Same operands through the LDS-DMA kernel (aligned view) and the register-staged kernel (the same
     values at a 1-byte offset, which forces the unaligned path): identical accumulation order, identical bits."""
