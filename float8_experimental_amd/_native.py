@@ -280,6 +280,10 @@ def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, produc
     if amax_out is not None:
         assert amax_out.dtype == torch.float32 and amax_out.numel() == 1 and amax_out.device == x.device
     _check_device(x.device)
+    if rows * cols == 0:  # nothing to convert (an empty batch); torch hands out null pointers for empty tensors
+        if amax_out is not None:
+            amax_out.zero_()
+        return out, out_t
     rc = lib().f8mi_cast_layout(xs.data_ptr(), rows, cols, ld, _DT[x.dtype], scale.data_ptr(), _DT[product_dtype],
                                 _F8[float8_dtype], out.data_ptr() if out is not None else None, int(out_kblock),
                                 out_t.data_ptr() if out_t is not None else None, int(out_t_kblock),

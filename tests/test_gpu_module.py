@@ -250,6 +250,37 @@ def test_single_copy_path_with_one_gradient_not_needed(f8, frozen):
     assert outs[0][1 if frozen == "input" else 2] is None
 
 
+@pytest.mark.parametrize("scaling", [("dyn", "dyn", "dyn"), ("del", "del", "del")])
+@pytest.mark.parametrize("k,n", [(384, 512), (100, 36)])
+def test_empty_batch(f8, scaling, k, n):
+    """No tokens: empty outputs, zero weight gradient, nothing launched on null pointers.  (The reference raises
+    inside torch.max on an empty tensor; an empty amax is defined as 0 here.)"""
+    torch.manual_seed(8)
+    lin = nn.Linear(k, n, bias=True).to(torch.bfloat16)
+    mod = f8.Float8Linear.from_float(lin, config=_cfg(f8, *scaling)).to(DEV)
+    for shape, fwd in (((0, k), mod.forward), ((2, 0, k), mod.forward), ((0, k), mod.forward_composed)):
+        if "del" in scaling:
+            f8.sync_float8_amax_and_scale_history(mod)
+        x = torch.randn(shape, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+        mod.weight.grad = mod.bias.grad = None
+        y = fwd(x)
+        assert y.shape == (*shape[:-1], n) and y.dtype == torch.bfloat16
+        y.backward(torch.randn(y.shape, device=DEV, dtype=torch.bfloat16))
+        assert x.grad.shape == x.shape
+        assert mod.weight.grad.shape == (n, k) and not mod.weight.grad.any()
+    # and the layer still works afterwards (delayed scaling: one batch later, once a real amax is in the history --
+    # the scales after empty batches come from amax = 0 and saturate everything, as delayed scaling will)
+    from oracle import torch_oracle as to
+
+    x = torch.randn(8, k, device=DEV, dtype=torch.bfloat16)
+    want = torch.nn.functional.linear(x, mod.weight, mod.bias)
+    for _ in range(2 if "del" in scaling else 1):
+        if "del" in scaling:
+            f8.sync_float8_amax_and_scale_history(mod)
+        got = mod(x)
+    assert to.sqnr(want.detach().cpu(), got.detach().cpu()) > 18.0
+
+
 # --------------------------------------------------------------- scales computed ahead of the forward
 
 
