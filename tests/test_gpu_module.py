@@ -281,6 +281,54 @@ def test_empty_batch(f8, scaling, k, n):
     assert to.sqnr(want.detach().cpu(), got.detach().cpu()) > 18.0
 
 
+def test_two_host_threads_on_their_own_streams(f8):
+    """The library keeps no mutable state between calls except what the caller hands it (workspace per stream):
+    two threads stepping their own layers on their own streams get the results of running alone."""
+    import threading
+
+    torch.manual_seed(9)
+    shapes = [(384, 512, 640), (200, 448, 96)]
+    mods, xs, dys, want = [], [], [], []
+    for m, k, n in shapes:
+        lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
+        mods.append(f8.Float8Linear.from_float(lin).to(DEV))
+        xs.append(torch.randn(m, k, device=DEV, dtype=torch.bfloat16))
+        dys.append(torch.randn(m, n, device=DEV, dtype=torch.bfloat16))
+
+    def run(i, out):
+        x = xs[i].clone().requires_grad_()
+        y = mods[i](x)
+        gx, gw = torch.autograd.grad(y, [x, mods[i].weight], dys[i])
+        out.append((y.detach(), gx, gw))
+
+    for i in range(2):
+        run(i, want)
+    torch.cuda.synchronize()
+    got = [[], []]
+    errors = []
+
+    def worker(i):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for _ in range(25):
+                    run(i, got[i])
+                torch.cuda.current_stream().synchronize()
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        assert len(got[i]) == 25
+        for trio in got[i]:
+            for a, b in zip(trio, want[i]):
+                assert torch.equal(a, b)
+
+
 # --------------------------------------------------------------- scales computed ahead of the forward
 
 
