@@ -1,4 +1,4 @@
-// K3 for few rows (m <= 128): C[m][n] = sum_k A[m][k] * Bt[n][k] where reading Bt once from HBM is all the
+// K3 for few rows (m <= 256): C[m][n] = sum_k A[m][k] * Bt[n][k] where reading Bt once from HBM is all the
 // work there is (a decode step of an inference linear: A is a handful of tokens, Bt the weight).
 //
 // The 256 x 256 tile kernels would put n / 256 workgroups on 256 CUs and walk the whole k on each, which is
@@ -12,8 +12,9 @@
 //
 // Operands are addressed as (row stride, stride of a 64-deep k block): row-major (ld, 64) or k-blocked
 // (64, rows * 64).  Needs k % 128 == 0 and 16-byte aligned operands and strides; any n.  Up to 64 rows of A go
-// through one workgroup per 32 columns; up to 128 rows are split into two such passes over Bt (second grid
-// dimension), which still beats the tile kernels' latency.
+// through one workgroup per 32 columns in tiles of 16, 32 or 64 rows; more rows in blocks of 128 (second grid
+// dimension: one pass over Bt per block, one step in flight per wave), which still beats the tile kernels'
+// latency up to 256 rows (k-blocked operands; row-major ones break even there).
 #include "f8mi_gemm_util.h"
 
 namespace f8mi {
@@ -24,7 +25,7 @@ constexpr int SK_WAVES = 8;
 constexpr int SK_THREADS = SK_WAVES * 64;
 constexpr int SK_NT = 2;     // 16-column tiles per workgroup
 // 128-deep steps loaded before the first is multiplied: four where the A fragments leave registers for it
-constexpr int sk_depth(int mt) { return mt <= 2 ? 4 : 2; }
+constexpr int sk_depth(int mt) { return mt <= 2 ? 4 : mt <= 4 ? 2 : 1; }
 
 __device__ __forceinline__ v8i load_frag_global(const uint8_t* p) {
     const uint4 lo = *(const uint4*)p;
@@ -137,7 +138,11 @@ static int launch_skinny3(dim3 g, hipStream_t stream, const uint8_t* A, int64_t 
                           int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
                           const void* bias) {
     const dim3 b(SK_THREADS);
-    if (M > 64) g.y = (unsigned)((M + 63) / 64);  // Bt is read once per 64 rows of A
+    if (M > 64) {  // blocks of 128 rows: Bt is read once per block (second grid dimension)
+        g.y = (unsigned)((M + 127) / 128);
+        hipLaunchKernelGGL((gemm_skinny_kernel<AF, BF, C_DT, 8>), g, b, 0, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias);
+        return check_hip(hipGetLastError(), "skinny gemm kernel launch");
+    }
     if (M <= 16) hipLaunchKernelGGL((gemm_skinny_kernel<AF, BF, C_DT, 1>), g, b, 0, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias);
     else if (M <= 32) hipLaunchKernelGGL((gemm_skinny_kernel<AF, BF, C_DT, 2>), g, b, 0, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias);
     else hipLaunchKernelGGL((gemm_skinny_kernel<AF, BF, C_DT, 4>), g, b, 0, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias);
@@ -153,7 +158,7 @@ static int launch_skinny2(int c_dtype, dim3 g, hipStream_t stream, const uint8_t
     return launch_skinny3<AF, BF, F8MI_FP32>(g, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias);
 }
 
-// Host side has checked: 1 <= M <= SKINNY_MAX_M (more than 64 rows: one pass over Bt per 64), K % 128 == 0, K >= 128, 16-byte aligned operands and strides.
+// Host side has checked: 1 <= M <= SKINNY_MAX_M, K % 128 == 0, K >= 128, 16-byte aligned operands and strides.
 int launch_gemm_skinny(int a_fmt, int b_fmt, int c_dtype, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                        const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                        int64_t ldc, const void* bias) {

@@ -162,8 +162,9 @@ static int allow_big_lds(K kern, int bytes, std::atomic<uint64_t>& done_mask) {
 
 // The 16x16x128 kernel with Bt (nt) or both operands (tt) given transposed: memory holds [contraction][rows];
 // lda / ldb = bytes between contraction rows, a_unit / b_unit = bytes between blocks of 64 rows.
-// few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands
-constexpr int SKINNY_MAX_M = 128;
+// few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands.  One limit for row-major and
+// k-blocked operands, so that the two entry points keep giving the same bits.
+constexpr int SKINNY_MAX_M = 256;
 int launch_gemm_skinny(int a_fmt, int b_fmt, int c_dtype, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                        const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                        int64_t ldc, const void* bias);

@@ -132,8 +132,8 @@ int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtyp
  * (float8_ops.py:158-190).  Both operands are contiguous along k (A row-major,
  * B column-major in the reference's words): forward x*W^T, grad_input dY*W and
  * grad_weight dY^T*x all have this form once the transposed copies exist.
- * Any m, n, k >= 0 is accepted (ragged edges are handled in the kernel).  Up to 128 rows of A with
- * k % 128 == 0 take a kernel that reads Bt once at memory speed (an inference decode step); it sums the
+ * Any m, n, k >= 0 is accepted (ragged edges are handled in the kernel).  Up to 256 rows of A with
+ * k % 128 == 0 take a kernel that reads Bt at memory speed (an inference decode step); it sums the
  * products in another order than the tile kernels, so its results agree with theirs within the
  * accumulation tolerance, not bit for bit.
  *   a_fmt/b_fmt   F8MI_E4M3FN / F8MI_E5M2 per operand
@@ -179,7 +179,7 @@ int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t
  * Forward x*W^T takes (0, 0); grad_input dY*W takes a = dY8 [n_out/64][tokens][64] (0) and bt = the forward's
  * W8 [k_in/64][n_out][64] (1); grad_weight dY^T*x takes a = that dY8 (1) and bt = the forward's x8 (1).
  * (1, 0) is not built.  Transposed operands need k % 128 == 0, k >= 384 and the operand's row count (m or n)
- * to be a multiple of 64.  Same result bits as f8mi_gemm_nt on the row-major operands (for m > 128: the
+ * to be a multiple of 64.  Same result bits as f8mi_gemm_nt on the row-major operands (for m > 256: the
  * few-row kernel of f8mi_gemm_nt is not used for transposed operands). */
 int f8mi_gemm_kb_ex(const void* a, int a_fmt, int a_transposed, const void* bt, int b_fmt, int b_transposed, int64_t m,
                     int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
