@@ -3,10 +3,11 @@
 //
 // The 256 x 256 tile kernels would put n / 256 workgroups on 256 CUs and walk the whole k on each, which is
 // 70 us for k = n = 8192 whatever m is.  Here a workgroup of eight waves owns 32 columns of C (two 16-row tiles
-// of Bt) and ALL rows of A; the waves split k among themselves, eight ways, and each streams its part of Bt
-// straight from memory into MFMA operands: a lane's operand of v_mfma_f32_16x16x128_f8f6f4 is 32 consecutive k
-// bytes of one row, two 16-byte loads, no LDS on the way.  Four steps of 128 k are loaded back to back before
-// the first is multiplied (16 loads of 16 bytes per lane in flight for Bt alone).  The A fragments come the same
+// of Bt) and all rows of A (of its block of A, past 64 rows); the waves split k among themselves, eight ways, and
+// each streams its part of Bt straight from memory into MFMA operands: a lane's operand of
+// v_mfma_f32_16x16x128_f8f6f4 is 32 consecutive k bytes of one row, two 16-byte loads, no LDS on the way.  With up
+// to 32 rows of A four steps of 128 k are loaded back to back before the first is multiplied (16 loads of 16
+// bytes per lane in flight for Bt alone), with more rows two or one.  The A fragments come the same
 // way (A is small and stays in the L2).  At the end the eight partial sums meet in LDS, are added in a
 // fixed order, scaled, biased, converted and stored.
 //
