@@ -236,10 +236,15 @@ KB = 64          # depth of one block of the k-blocked operand layout
 KB_MIN_K = 384   # shortest contraction the k-blocked GEMM takes
 
 
-def tn_ok(*dims: int) -> bool:
-    """True if every dimension of a linear layer (tokens, in_features, out_features) allows the GEMMs to read
-    one k-blocked copy per tensor, transposed where needed (f8mi_gemm_kb_ex): multiples of 128, at least 384."""
-    return all(d % 128 == 0 and d >= KB_MIN_K for d in dims)
+def tn_ok(m: int, k: int, n: int) -> bool:
+    """True if a linear layer with m tokens, k in_features and n out_features should keep one k-blocked fp8 copy per
+    tensor and let the backward GEMMs read it transposed (f8mi_gemm_kb_ex): every dimension a multiple of 128 and at
+    least 384 -- and grad_input and grad_weight large enough for the 256 x 256-tile kernels, the only ones that read
+    transposed operands (smaller outputs are faster from transposed copies through the 128 x 128-tile kernel)."""
+    if not all(d % 128 == 0 and d >= KB_MIN_K for d in (m, k, n)):
+        return False
+    tiles = lambda rows, cols: -(-rows // 256) * -(-cols // 256)
+    return tiles(m, k) > 64 and tiles(n, k) > 64
 
 
 def kblock_ok(k: int) -> bool:

@@ -203,12 +203,15 @@ def test_fused_forward_equals_the_composed_reference_pipeline(f8, scaling):
 
 @pytest.mark.parametrize("scaling", [("dyn", "dyn", "dyn"), ("del", "del", "del")])
 @pytest.mark.parametrize("m,k,n", [(512, 384, 448), (384, 512, 200), (100, 448, 384), (448, 200, 640),
-                                   (512, 384, 640), (384, 768, 512), (1152, 640, 384)])
+                                   (512, 384, 640), (384, 768, 512), (2304, 2048, 2304), (4352, 4096, 4224)])
 def test_fused_path_with_k_blocked_operands_equals_the_composed_pipeline(f8, scaling, m, k, n):
     """Sizes at which some or all of the three GEMMs take k-blocked operands (contraction a multiple
     of 64 and >= 384), and sizes at which every tensor is cast once and read transposed by the GEMM that
-    contracts its other dimension (all three multiples of 128), against the composed, row-major
-    pipeline: identical bits everywhere."""
+    contracts its other dimension (the last two: all three multiples of 128 and every product of more than 64
+    tiles of 256 x 256), against the composed, row-major pipeline: identical bits everywhere."""
+    from float8_experimental_amd import _native
+
+    assert _native.tn_ok(m, k, n) == (m >= 2304)
     torch.manual_seed(2)
     lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
     a = f8.Float8Linear.from_float(copy.deepcopy(lin), config=_cfg(f8, *scaling)).to(DEV)
@@ -232,7 +235,7 @@ def test_fused_path_with_k_blocked_operands_equals_the_composed_pipeline(f8, sca
 @pytest.mark.parametrize("frozen", ["weight", "input"])
 def test_single_copy_path_with_one_gradient_not_needed(f8, frozen):
     torch.manual_seed(4)
-    m, k, n = 384, 512, 640
+    m, k, n = 2304, 2048, 2432  # one fp8 copy per tensor, read transposed in backward
     lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
     a = f8.Float8Linear.from_float(copy.deepcopy(lin)).to(DEV)
     b = f8.Float8Linear.from_float(copy.deepcopy(lin)).to(DEV)
