@@ -311,8 +311,8 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     const int M = (int)m, N = (int)n, K = (int)k;
     if (aligned && M <= SKINNY_MAX_M && K % 128 == 0 && K > 0 && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
-    if (aligned && use_mid_tiles(tiles_m * tiles_n, K) && gemm_impl() == 0)
-        return launch_gemm_mid(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
+    if (const int mid = (aligned && gemm_impl() == 0) ? use_mid_tiles(tiles_m * tiles_n, K) : 0)
+        return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
     // F8MI_GEMM_IMPL=staged forces the register-staged kernel, =dma32 the 32x32x64 LDS-DMA kernel (comparison runs)
     if (aligned && K >= 384 && K % 64 == 0 && gemm_impl() != 1) {
         if (K % 128 == 0 && gemm_impl() != 2)
@@ -345,8 +345,8 @@ extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_f
     if (m <= SKINNY_MAX_M && k % 128 == 0 && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n,
                                   (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
-    if (use_mid_tiles(tiles_m * tiles_n, k) && gemm_impl() == 0)
-        return launch_gemm_mid(a_fmt, b_fmt, c_dtype, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n, (int)k,
+    if (const int mid = gemm_impl() == 0 ? use_mid_tiles(tiles_m * tiles_n, k) : 0)
+        return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n, (int)k,
                                scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
     if (k % 128 == 0 && gemm_impl() != 2)
         return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,

@@ -163,13 +163,18 @@ static int allow_big_lds(K kern, int bytes, std::atomic<uint64_t>& done_mask) {
 
 // The 16x16x128 kernel with Bt (nt) or both operands (tt) given transposed: memory holds [contraction][rows];
 // lda / ldb = bytes between contraction rows, a_unit / b_unit = bytes between blocks of 64 rows.
-// 128 x 128-tile kernel (f8mi_gemm_mid.hip) for outputs of few 256 x 256 tiles: K % 128 == 0, aligned operands
-int launch_gemm_mid(int a_fmt, int b_fmt, int c_dtype, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
+// 128-row-tile kernels (f8mi_gemm_mid.hip) for outputs of few 256 x 256 tiles: K % 128 == 0, aligned operands.
+// wide = false: 128 x 128 tiles, true: 128 x 256.
+int launch_gemm_mid(int a_fmt, int b_fmt, int c_dtype, bool wide, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                     const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                     int64_t ldc, const void* bias, int c_vec_ok);
-// it takes over when the 256 x 256 tiles would leave three quarters of the CUs without one (its own 128 x 128 tiles
-// then number at most one per CU; with more, the large tiles win again: measured)
-inline bool use_mid_tiles(int64_t tiles_256, int64_t k) { return tiles_256 <= MID_MAX_TILES_256 && k % 128 == 0 && k >= 128; }
+// They take over while their own tiles number at most one per CU: up to 64 tiles of 256 x 256 the 128 x 128 ones,
+// up to 128 the 128 x 256 ones (with more, the large tiles win again: measured).
+// Returns 0: large tiles, 1: 128 x 128, 2: 128 x 256.
+inline int use_mid_tiles(int64_t tiles_256, int64_t k) {
+    if (k % 128 != 0 || k < 128 || tiles_256 > 2 * MID_MAX_TILES_256) return 0;
+    return tiles_256 <= MID_MAX_TILES_256 ? 1 : 2;
+}
 // few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands.  One limit for row-major and
 // k-blocked operands, so that the two entry points keep giving the same bits.
 constexpr int SKINNY_MAX_M = 256;

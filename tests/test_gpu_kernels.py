@@ -396,16 +396,17 @@ def test_gemm_few_rows_kblocked_equals_row_major_bitwise(nat, m, n, k):
     assert torch.equal(sub, want[: max(1, m // 3)])
 
 
-# Outputs of few 256 x 256 tiles (at most 64 of them, more than 256 rows, k % 128 == 0) take the 128 x 128-tile kernel.
+# Outputs of few 256 x 256 tiles (more than 256 rows, k % 128 == 0) take the 128 x 128-tile kernel (at most 64 of them) or
+# the 128 x 256-tile kernel (65 to 128; the last three cases).
 @pytest.mark.parametrize("m,n,k", [(257, 128, 128), (300, 520, 1024), (512, 1000, 256), (1024, 2048, 640), (384, 8192, 2048),
-                                   (4099, 500, 1152)])
+                                   (4099, 500, 1152), (1024, 8192, 1024), (1000, 5000, 384), (2049, 3000, 128)])
 @pytest.mark.parametrize("out_dt", [torch.bfloat16, torch.float32])
 def test_gemm_mid_tile_kernel_shapes(nat, m, n, k, out_dt):
     fm = [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2"), ("e5m2", "e5m2")][(m + n + k // 128) % 4]
     _gemm_check(nat, m, n, k, fm[0], fm[1], out_dt, seed=m + n + k, bias=(n % 2 == 0))
 
 
-@pytest.mark.parametrize("m,n,k", [(300, 520, 1024), (1000, 264, 2048), (512, 1024, 384)])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 1024), (1000, 264, 2048), (512, 1024, 384), (1100, 4500, 640)])
 def test_gemm_mid_tile_kernel_equals_the_large_tile_kernel_bitwise(nat, m, n, k):
     """The same rows of A inside a matrix tall enough for the 256 x 256-tile kernel: identical bits (same accumulation
     order), row-major and k-blocked."""
@@ -413,7 +414,7 @@ def test_gemm_mid_tile_kernel_equals_the_large_tile_kernel_bitwise(nat, m, n, k)
     bt = _rand_fp8((n, k), torch.float8_e4m3fn, n + k, 4.0).to(DEV)
     sa, sb = torch.tensor(2.0, device=DEV), torch.tensor(0.25, device=DEV)
     bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 3).to(torch.bfloat16).to(DEV)
-    tall = 256 * (64 // ((n + 255) // 256) + 2)
+    tall = 256 * (128 // ((n + 255) // 256) + 2)
     a_tall = torch.cat([a.view(torch.uint8), torch.zeros(tall - m, k, dtype=torch.uint8, device=DEV)]).view(a.dtype)
     for out_dt, b in ((torch.bfloat16, bias), (torch.float32, None)):
         want = nat.gemm_nt(a_tall, sa, bt, sb, out_dt, bias=b)[:m]
