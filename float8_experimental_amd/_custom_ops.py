@@ -23,10 +23,7 @@ def _layout(t_rows: int, t_cols: int, kblock: bool):
 
 
 def _cast_dynamic(t2d, float8_dtype, want_row, want_t, row_kb, t_kb):
-    _, scale = _native.amax_scale(t2d, float8_dtype, want_amax=False)
-    row, tr = _native.cast(t2d, scale, float8_dtype, product_dtype=t2d.dtype, want_out=want_row, want_out_t=want_t,
-                           out_kblock=row_kb, out_t_kblock=t_kb)
-    return row, tr, scale
+    return _native.cast_dynamic(t2d, float8_dtype, want_out=want_row, want_out_t=want_t, out_kblock=row_kb, out_t_kblock=t_kb)
 
 
 def _gemm(a8, sa, b8, sb, out_dtype, kb):

@@ -33,6 +33,7 @@ EXPORTS = (
     "f8mi_amax_tile_elems",
     "f8mi_cast",
     "f8mi_cast_layout",
+    "f8mi_cast_dynamic",
     "f8mi_gemm_nt",
     "f8mi_gemm_nt_kb",
     "f8mi_gemm_kb_ex",
@@ -85,6 +86,8 @@ def lib() -> C.CDLL:
         L.f8mi_cast.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, vp, fp, vp, vp]
         L.f8mi_cast_layout.restype = i32
         L.f8mi_cast_layout.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, i32, vp, i32, fp, vp]
+        L.f8mi_cast_dynamic.restype = i32
+        L.f8mi_cast_dynamic.argtypes = [vp, i64, i64, i64, i32, i32, fp, vp, i32, vp, i32, vp, vp]
         L.f8mi_gemm_nt_kb.restype = i32
         L.f8mi_gemm_nt_kb.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_kb_ex.restype = i32
@@ -295,6 +298,36 @@ def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, produc
                                 amax_out.data_ptr() if amax_out is not None else None, _stream(x))
     _check(rc, "f8mi_cast_layout")
     return out, out_t
+
+
+def cast_dynamic(x: torch.Tensor, float8_dtype: torch.dtype, want_out: bool = True, want_out_t: bool = False,
+                 out_kblock: bool = False, out_t_kblock: bool = False):
+    """(out, out_t, scale): ``amax_scale`` in x's dtype followed by ``cast`` with that scale, as one library call
+    (hp_tensor_to_float8_dynamic of the reference); small tensors take a single launch.  See f8mi_cast_dynamic."""
+    _require_gpu(x, "x")
+    xs, rows, cols, ld = _as_2d(x)
+    scale = torch.empty((), dtype=torch.float32, device=x.device)
+    out = out_t = None
+    if want_out:
+        if out_kblock:
+            assert cols % KB == 0, f"k-blocked out needs cols % {KB} == 0, got {cols}"
+            out = torch.empty((cols // KB, rows, KB), dtype=float8_dtype, device=x.device)
+        else:
+            out = torch.empty(x.shape, dtype=float8_dtype, device=x.device)
+    if want_out_t:
+        if out_t_kblock:
+            assert rows % KB == 0, f"k-blocked out_t needs rows % {KB} == 0, got {rows}"
+            out_t = torch.empty((rows // KB, cols, KB), dtype=float8_dtype, device=x.device)
+        else:
+            out_t = torch.empty((cols, rows), dtype=float8_dtype, device=x.device)
+    ws = workspace(x.device)
+    empty = rows * cols == 0  # torch hands out null pointers for empty tensors: only the scale is computed
+    rc = lib().f8mi_cast_dynamic(xs.data_ptr() if not empty else None, rows, cols, ld, _DT[x.dtype], _F8[float8_dtype],
+                                 scale.data_ptr(), out.data_ptr() if out is not None and not empty else None, int(out_kblock),
+                                 out_t.data_ptr() if out_t is not None and not empty else None, int(out_t_kblock),
+                                 ws.data_ptr(), _stream(x))
+    _check(rc, "f8mi_cast_dynamic")
+    return out, out_t, scale
 
 
 def gemm_nt_kb(a_kb: torch.Tensor, a_scale: torch.Tensor, bt_kb: torch.Tensor, b_scale: torch.Tensor,

@@ -255,6 +255,86 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
     }
 }
 
+// Dynamic scaling of a small tensor in ONE launch: amax, scale and cast by a single workgroup (the tensor is
+// read twice, the second time from the L2).  Same arithmetic, element for element, as amax kernel + cast kernel;
+// it exists because three or four launches cost more than the work when the tensor is a few rows of activations.
+constexpr int SMALL_THREADS = 1024;
+constexpr int64_t SMALL_MAX_BYTES = 256 * 1024;
+
+template <int DT, int FMT, bool VEC>
+__global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
+                                                                           int64_t ld, float* __restrict__ scale_out,
+                                                                           uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
+                                                                           int out_kb, int out_t_kb) {
+    __shared__ uint32_t red[SMALL_THREADS / 64];
+    __shared__ uint32_t amax_bits;
+    const int t = threadIdx.x;
+    const int64_t groups = (cols + 7) / 8, items = rows * groups;  // an item: eight consecutive elements of a row
+    uint32_t m = 0;
+    for (int64_t it = t; it < items; it += SMALL_THREADS) {
+        Row8<DT> r;
+        load_row8<DT, VEC>(r, x, it / groups, (it % groups) * 8, rows, cols, ld);
+        m = absmax_row<DT>(r, m);
+    }
+    m = wave_max_u32(m);
+    if ((t & 63) == 0) red[t >> 6] = m;
+    __syncthreads();
+    if (t < 64) {
+        uint32_t v = t < SMALL_THREADS / 64 ? red[t] : 0u;
+        v = wave_max_u32(v);
+        if (t == 0) amax_bits = v;
+    }
+    __syncthreads();
+    // the scale in the tensor's own dtype, as tensor_to_scale computes it (fp16 tensors: clamped to 65504)
+    const float scale = amax_to_scale_dev(abs_bits_to_float(amax_bits, DT), DT, FMT, DT == F8MI_FP16);
+    if (t == 0) *scale_out = scale;
+    constexpr float fmax = FMT == F8MI_E4M3FN ? 448.0f : 57344.0f;
+    const bool out_vec = (cols % 8 == 0) && ((uintptr_t)out % 8 == 0);
+    for (int64_t it = t; it < items; it += SMALL_THREADS) {
+        const int64_t row = it / groups, col = (it % groups) * 8;
+        Row8<DT> r;
+        load_row8<DT, VEC>(r, x, row, col, rows, cols, ld);
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) scale_clamp2<DT>(elem<DT>(r, i), elem<DT>(r, i + 1), scale, fmax, f[i], f[i + 1]);
+        const uint32_t lo = cvt4_fp8<FMT>(f[0], f[1], f[2], f[3]), hi = cvt4_fp8<FMT>(f[4], f[5], f[6], f[7]);
+        if (out) {
+            uint8_t* p = out_kb ? out + ((col >> 6) * rows + row) * 64 + (col & 63) : out + row * cols + col;
+            if (out_vec) {
+                *(uint2*)p = make_uint2(lo, hi);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    if (col + i < cols) p[i] = (uint8_t)((i < 4 ? lo >> (8 * i) : hi >> (8 * (i - 4))) & 0xffu);
+            }
+        }
+        if (out_t) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int64_t c = col + i;
+                if (c < cols) {
+                    uint8_t* p = out_t_kb ? out_t + ((row >> 6) * cols + c) * 64 + (row & 63) : out_t + c * rows + row;
+                    *p = (uint8_t)((i < 4 ? lo >> (8 * i) : hi >> (8 * (i - 4))) & 0xffu);
+                }
+            }
+        }
+    }
+}
+
+template <int DT>
+static int launch_cast_small(int fmt, bool vec, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
+                             float* scale_dev, uint8_t* out, uint8_t* out_t, int out_kb, int out_t_kb) {
+    const dim3 g(1), b(SMALL_THREADS);
+    if (fmt == F8MI_E4M3FN) {
+        if (vec) hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E4M3FN, true>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+        else hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E4M3FN, false>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+    } else {
+        if (vec) hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E5M2, true>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+        else hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E5M2, false>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+    }
+    return check_hip(hipGetLastError(), "cast (dynamic, one workgroup) kernel launch");
+}
+
 __global__ void cast_zero_amax_kernel(float* amax_out) {
     if (threadIdx.x == 0) *amax_out = 0.0f;
 }
@@ -330,4 +410,28 @@ extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, 
     (void)workspace;
     return f8mi_cast_layout(x, rows, cols, ld, in_dtype, scale_dev, product_dtype, fp8_fmt, out, F8MI_LAYOUT_ROWMAJOR, out_t,
                             F8MI_LAYOUT_ROWMAJOR, amax_dev, stream);
+}
+
+extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt, float* scale_dev,
+                                 uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout, void* workspace, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!scale_dev) { set_error("f8mi_cast_dynamic: null scale"); return F8MI_ERR_INVALID_ARG; }
+    if (rows < 0 || cols < 0 || ld < cols || in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast_dynamic: bad shape or dtype/format code"); return F8MI_ERR_INVALID_ARG; }
+    const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
+    const int64_t n = rows * cols;
+    if (n > 0 && (int64_t)(n * esz) <= SMALL_MAX_BYTES && (out || out_t)) {
+        if ((out_layout != F8MI_LAYOUT_ROWMAJOR && out_layout != F8MI_LAYOUT_KBLOCK64) || (out_t_layout != F8MI_LAYOUT_ROWMAJOR && out_t_layout != F8MI_LAYOUT_KBLOCK64)) { set_error("f8mi_cast_dynamic: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
+        if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast_dynamic: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
+        if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast_dynamic: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
+        if (!x) { set_error("f8mi_cast_dynamic: null tensor"); return F8MI_ERR_INVALID_ARG; }
+        const bool vec = ((uintptr_t)x % 16 == 0) && ((ld * esz) % 16 == 0);
+        const int out_kb = out_layout == F8MI_LAYOUT_KBLOCK64, out_t_kb = out_t_layout == F8MI_LAYOUT_KBLOCK64;
+        ProfScope prof(F8MI_K_CAST, (double)n * (2 * esz + (out ? 1 : 0) + (out_t ? 1 : 0)), stream);
+        if (in_dtype == F8MI_BF16) return launch_cast_small<F8MI_BF16>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+        if (in_dtype == F8MI_FP16) return launch_cast_small<F8MI_FP16>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+        return launch_cast_small<F8MI_FP32>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+    }
+    int rc = f8mi_amax_scale(x, rows, cols, ld, in_dtype, fp8_fmt, in_dtype, in_dtype == F8MI_FP16, nullptr, scale_dev, workspace, stream_);
+    if (rc || n == 0 || (!out && !out_t)) return rc;
+    return f8mi_cast_layout(x, rows, cols, ld, in_dtype, scale_dev, in_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, nullptr, stream_);
 }

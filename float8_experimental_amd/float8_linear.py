@@ -73,8 +73,8 @@ def _cast_for_gemm(t2d: torch.Tensor, float8_dtype, delayed: Optional[_DelayedBu
                    known_scale: Optional[torch.Tensor] = None):
     """fp8 copies of a 2-D tensor for the GEMMs: (as is, transposed, scale).
 
-    dynamic: one amax+scale launch, one cast launch (float8_utils.py:115-120 +
-    float8_tensor.py:158-159 of the reference); delayed: first-iteration init if needed,
+    dynamic: amax+scale, then the cast, in one library call (float8_utils.py:115-120 +
+    float8_tensor.py:158-159 of the reference; one launch for a small tensor); delayed: first-iteration init if needed,
     then ONE launch that casts with the existing scale and records this step's amax
     (float8_scaling_utils.py:65-125).  ``row_kb`` / ``t_kb`` ask for the k-blocked layout
     of the respective copy (same bytes, placed [k/64][rows][64] for the GEMM that contracts it).
@@ -82,13 +82,12 @@ def _cast_for_gemm(t2d: torch.Tensor, float8_dtype, delayed: Optional[_DelayedBu
     (``precompute_float8_dynamic_scale_for_fsdp``); the amax pass is skipped.
     """
     if delayed is None:
-        if known_scale is not None:
-            scale = known_scale
-        else:
-            _, scale = _native.amax_scale(t2d, float8_dtype, want_amax=False)
-        row, tr = _native.cast(t2d, scale, float8_dtype, product_dtype=t2d.dtype, want_out=want_row, want_out_t=want_t,
+        if known_scale is None:
+            return _native.cast_dynamic(t2d, float8_dtype, want_out=want_row, want_out_t=want_t, out_kblock=row_kb,
+                                        out_t_kblock=t_kb)
+        row, tr = _native.cast(t2d, known_scale, float8_dtype, product_dtype=t2d.dtype, want_out=want_row, want_out_t=want_t,
                                out_kblock=row_kb, out_t_kblock=t_kb)
-        return row, tr, scale
+        return row, tr, known_scale
     if not is_initialized:
         _native.amax_scale(t2d, float8_dtype, want_scale=False, amax_out=delayed.amax)
         _native.delayed_init(delayed.amax, delayed.history, delayed.scale, float8_dtype, t2d.dtype == torch.float16)

@@ -111,9 +111,9 @@ class Float8InferenceLinear(torch.nn.Linear):
         use_kb = _native.kblock_ok(k)
         if self.static_quantization_scale is not None:
             scale = self.static_quantization_scale
+            x8, _ = _native.cast(x2, scale, e4m3_dtype, product_dtype=_product_dtype(x2, scale), out_kblock=use_kb)
         else:
-            _, scale = _native.amax_scale(x2, e4m3_dtype, want_amax=False)
-        x8, _ = _native.cast(x2, scale, e4m3_dtype, product_dtype=_product_dtype(x2, scale), out_kblock=use_kb)
+            x8, _, scale = _native.cast_dynamic(x2, e4m3_dtype, out_kblock=use_kb)
         if use_kb:
             y = _native.gemm_nt_kb(x8, scale, self._weight_kblocked(), w._scale, out_dtype, bias=bias)
         else:

@@ -313,6 +313,39 @@ def test_golden_cast_fixtures_on_gpu(nat):
 # ------------------------------------------------------------------ K3 gemm
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(1, 8), (1, 8192), (3, 1000), (16, 8192), (64, 512), (37, 129), (128, 1024), (200, 700),
+                                   (5, 7, 64), (512, 4096)])
+def test_cast_dynamic_equals_amax_scale_then_cast(nat, dt, shape):
+    """f8mi_cast_dynamic (one workgroup up to 256 KB, the two kernels beyond): scale and bytes of every output layout
+    equal those of f8mi_amax_scale followed by f8mi_cast, bit for bit; NaN and all-zero tensors included."""
+    tdt = TORCH_DT[dt]
+    x = heavy(shape, tdt, 21).to(DEV)
+    variants = [x]
+    if len(shape) == 2 and shape[1] >= 64:
+        variants.append(x[:, 3:shape[1] - 2])          # unaligned, strided rows
+        z = torch.zeros_like(x)
+        variants.append(z)
+        n = x.clone()
+        n[-1, -1] = float("nan")
+        variants.append(n)
+    for v in variants:
+        rows, cols = v.reshape(-1, v.shape[-1]).shape
+        for fmt, (code, f8dt) in F8.items():
+            _, s_want = nat.amax_scale(v, f8dt, want_amax=False)
+            kb, tkb = cols % 64 == 0, rows % 64 == 0
+            for okb, otkb in {(False, False), (kb, tkb)}:
+                o_want, t_want = nat.cast(v, s_want, f8dt, want_out_t=True, out_kblock=okb, out_t_kblock=otkb)
+                o, t, s = nat.cast_dynamic(v, f8dt, want_out_t=True, out_kblock=okb, out_t_kblock=otkb)
+                assert s.view(torch.int32).item() == s_want.view(torch.int32).item() or (torch.isnan(s) and torch.isnan(s_want))
+                assert same_bytes_mod_nan_sign(fp8_bytes(o), fp8_bytes(o_want)), (dt, shape, fmt, okb)
+                assert same_bytes_mod_nan_sign(fp8_bytes(t), fp8_bytes(t_want)), (dt, shape, fmt, otkb)
+    o, t, s = nat.cast_dynamic(torch.empty(0, 64, device=DEV, dtype=tdt), torch.float8_e4m3fn, want_out_t=True)
+    assert o.shape == (0, 64) and t.shape == (64, 0)
+    _, s_want = nat.amax_scale(torch.empty(0, 64, device=DEV, dtype=tdt), torch.float8_e4m3fn)
+    assert s.item() == s_want.item()
+
+
 def _rand_fp8(shape, tdt, seed, scale=1.0):
     g = torch.Generator().manual_seed(seed)
     v = torch.randn(shape, generator=g) * scale
