@@ -255,11 +255,13 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
     }
 }
 
-// Dynamic scaling of a small tensor in ONE launch: amax, scale and cast by a single workgroup (the tensor is
-// read twice, the second time from the L2).  Same arithmetic, element for element, as amax kernel + cast kernel;
-// it exists because three or four launches cost more than the work when the tensor is a few rows of activations.
+// Dynamic scaling of a small tensor in ONE launch: amax, scale and cast by a single workgroup that holds the whole
+// tensor in registers (at most four items of eight elements per lane, loaded back to back).  Same arithmetic,
+// element for element, as amax kernel + cast kernel; it exists because three or four launches cost more than
+// the work when the tensor is a few rows of activations.
 constexpr int SMALL_THREADS = 1024;
-constexpr int64_t SMALL_MAX_BYTES = 256 * 1024;
+constexpr int SMALL_ITEMS_PER_THREAD = 4;
+constexpr int64_t SMALL_MAX_ITEMS = (int64_t)SMALL_THREADS * SMALL_ITEMS_PER_THREAD;  // 32 K elements: 64 KB of bf16
 
 template <int DT, int FMT, bool VEC>
 __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
@@ -270,12 +272,16 @@ __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const
     __shared__ uint32_t amax_bits;
     const int t = threadIdx.x;
     const int64_t groups = (cols + 7) / 8, items = rows * groups;  // an item: eight consecutive elements of a row
+    Row8<DT> r[SMALL_ITEMS_PER_THREAD];
     uint32_t m = 0;
-    for (int64_t it = t; it < items; it += SMALL_THREADS) {
-        Row8<DT> r;
-        load_row8<DT, VEC>(r, x, it / groups, (it % groups) * 8, rows, cols, ld);
-        m = absmax_row<DT>(r, m);
+#pragma unroll
+    for (int u = 0; u < SMALL_ITEMS_PER_THREAD; u++) {
+        const int64_t it = t + (int64_t)u * SMALL_THREADS;
+        // past the last item: row == rows, which load_row8 reads as zeros
+        load_row8<DT, VEC>(r[u], x, it < items ? it / groups : rows, (it % groups) * 8, rows, cols, ld);
     }
+#pragma unroll
+    for (int u = 0; u < SMALL_ITEMS_PER_THREAD; u++) m = absmax_row<DT>(r[u], m);
     m = wave_max_u32(m);
     if ((t & 63) == 0) red[t >> 6] = m;
     __syncthreads();
@@ -290,13 +296,14 @@ __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const
     if (t == 0) *scale_out = scale;
     constexpr float fmax = FMT == F8MI_E4M3FN ? 448.0f : 57344.0f;
     const bool out_vec = (cols % 8 == 0) && ((uintptr_t)out % 8 == 0);
-    for (int64_t it = t; it < items; it += SMALL_THREADS) {
+#pragma unroll
+    for (int u = 0; u < SMALL_ITEMS_PER_THREAD; u++) {
+        const int64_t it = t + (int64_t)u * SMALL_THREADS;
+        if (it >= items) continue;
         const int64_t row = it / groups, col = (it % groups) * 8;
-        Row8<DT> r;
-        load_row8<DT, VEC>(r, x, row, col, rows, cols, ld);
         float f[8];
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) scale_clamp2<DT>(elem<DT>(r, i), elem<DT>(r, i + 1), scale, fmax, f[i], f[i + 1]);
+        for (int i = 0; i < 8; i += 2) scale_clamp2<DT>(elem<DT>(r[u], i), elem<DT>(r[u], i + 1), scale, fmax, f[i], f[i + 1]);
         const uint32_t lo = cvt4_fp8<FMT>(f[0], f[1], f[2], f[3]), hi = cvt4_fp8<FMT>(f[4], f[5], f[6], f[7]);
         if (out) {
             uint8_t* p = out_kb ? out + ((col >> 6) * rows + row) * 64 + (col & 63) : out + row * cols + col;
@@ -419,14 +426,14 @@ extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int6
     if (rows < 0 || cols < 0 || ld < cols || in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast_dynamic: bad shape or dtype/format code"); return F8MI_ERR_INVALID_ARG; }
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
     const int64_t n = rows * cols;
-    if (n > 0 && (int64_t)(n * esz) <= SMALL_MAX_BYTES && (out || out_t)) {
+    if (n > 0 && rows * ((cols + 7) / 8) <= SMALL_MAX_ITEMS && (out || out_t)) {
         if ((out_layout != F8MI_LAYOUT_ROWMAJOR && out_layout != F8MI_LAYOUT_KBLOCK64) || (out_t_layout != F8MI_LAYOUT_ROWMAJOR && out_t_layout != F8MI_LAYOUT_KBLOCK64)) { set_error("f8mi_cast_dynamic: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
         if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast_dynamic: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
         if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast_dynamic: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
         if (!x) { set_error("f8mi_cast_dynamic: null tensor"); return F8MI_ERR_INVALID_ARG; }
         const bool vec = ((uintptr_t)x % 16 == 0) && ((ld * esz) % 16 == 0);
         const int out_kb = out_layout == F8MI_LAYOUT_KBLOCK64, out_t_kb = out_t_layout == F8MI_LAYOUT_KBLOCK64;
-        ProfScope prof(F8MI_K_CAST, (double)n * (2 * esz + (out ? 1 : 0) + (out_t ? 1 : 0)), stream);
+        ProfScope prof(F8MI_K_CAST, (double)n * (esz + (out ? 1 : 0) + (out_t ? 1 : 0)), stream);
         if (in_dtype == F8MI_BF16) return launch_cast_small<F8MI_BF16>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
         if (in_dtype == F8MI_FP16) return launch_cast_small<F8MI_FP16>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
         return launch_cast_small<F8MI_FP32>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);

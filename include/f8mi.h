@@ -168,8 +168,8 @@ int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int 
 /* Dynamic scaling in one call: scale = f8mi_amax_scale(x) in x's own dtype, then f8mi_cast_layout(x, scale) with the
  * product in x's dtype -- hp_tensor_to_float8_dynamic (float8_scaling_utils.py:33-62: tensor_to_scale, then
  * hp_tensor_and_scale_to_float8 with the 0-dim scale).  *scale_dev receives the scale.  A tensor of at most
- * 256 KB goes through one launch of one workgroup (a few rows of activations: the launches cost more than the
- * work), anything larger through the two kernels above; the results are the same bits either way.
+ * 32 K elements goes through one launch of one workgroup (a few rows of activations: the launches cost more
+ * than the work), anything larger through the two kernels above; the results are the same bits either way.
  * `workspace` as for f8mi_amax_scale. */
 int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt, float* scale_dev,
                       uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout, void* workspace, void* stream);

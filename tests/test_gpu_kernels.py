@@ -314,10 +314,10 @@ def test_golden_cast_fixtures_on_gpu(nat):
 
 
 @pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
-@pytest.mark.parametrize("shape", [(1, 8), (1, 8192), (3, 1000), (16, 8192), (64, 512), (37, 129), (128, 1024), (200, 700),
-                                   (5, 7, 64), (512, 4096)])
+@pytest.mark.parametrize("shape", [(1, 8), (1, 8192), (3, 1000), (4, 8192), (16, 8192), (64, 512), (37, 129), (128, 1024),
+                                   (200, 700), (5, 7, 64), (4096, 1), (4097, 3), (512, 4096)])
 def test_cast_dynamic_equals_amax_scale_then_cast(nat, dt, shape):
-    """f8mi_cast_dynamic (one workgroup up to 256 KB, the two kernels beyond): scale and bytes of every output layout
+    """f8mi_cast_dynamic (one workgroup up to 32 K elements, the two kernels beyond): scale and bytes of every output layout
     equal those of f8mi_amax_scale followed by f8mi_cast, bit for bit; NaN and all-zero tensors included."""
     tdt = TORCH_DT[dt]
     x = heavy(shape, tdt, 21).to(DEV)
