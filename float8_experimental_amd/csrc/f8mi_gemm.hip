@@ -309,6 +309,12 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     const uint8_t* A = (const uint8_t*)a;
     const uint8_t* B = (const uint8_t*)bt;
     const int M = (int)m, N = (int)n, K = (int)k;
+    // Which kernel (the k-blocked entry point below decides the same way, so both give the same bits):
+    //   aligned, K % 128 == 0:  up to 256 rows            -> few-row kernel (Bt streamed once, k split over waves)
+    //                           up to 64 / 128 large tiles -> 128 x 128 / 128 x 256 tiles
+    //                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA
+    //   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
+    //   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
     if (aligned && M <= SKINNY_MAX_M && K % 128 == 0 && K > 0 && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
     if (const int mid = (aligned && gemm_impl() == 0) ? use_mid_tiles(tiles_m * tiles_n, K) : 0)
