@@ -285,7 +285,7 @@ def test_cast_row_strided_and_c_oracle(nat):
 
 
 def test_cfg1_dy_ones(nat):
-    """BASELINE config 1: dY = ones -> scale 57344, every e5m2 byte 0x7B."""
+    """Benchmark configuration 1: dY = ones -> scale 57344, every e5m2 byte 0x7B."""
     dy = torch.ones(2048, 4096, dtype=torch.bfloat16, device=DEV)
     a, s = nat.amax_scale(dy, torch.float8_e5m2)
     assert a.item() == 1.0 and s.item() == 57344.0

@@ -376,7 +376,7 @@ def test_precomputed_weight_scales_give_the_same_step(f8, dt):
 
 
 def test_cfg1_against_the_reference_fixture(f8):
-    """BASELINE config 1: x[2048,4096] ~N(0,1), Linear(4096,4096) default init, seed 0, y.sum().backward()."""
+    """Benchmark configuration 1 (the reference's CPU-runnable case): x[2048,4096] ~N(0,1), Linear(4096,4096) default init, seed 0, y.sum().backward()."""
     import hashlib
 
     g = load("cfg1")
