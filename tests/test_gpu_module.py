@@ -232,6 +232,41 @@ def test_fused_path_with_k_blocked_operands_equals_the_composed_pipeline(f8, sca
             assert torch.equal(u, v)
 
 
+@pytest.mark.parametrize("scaling", [("dyn", "dyn", "dyn"), ("del", "del", "del")])
+def test_fp16_layer_fused_equals_composed_and_scales_stay_finite(f8, scaling):
+    """fp16 weights and activations: scales are computed in fp16 and clamped to 65504 (reference float8_utils.py:54-55,
+    test_base.py:566-586), also when the tensor is tiny; fused and composed routes agree bit for bit."""
+    from oracle import torch_oracle as to
+
+    torch.manual_seed(12)
+    m, k, n = 200, 448, 384
+    lin = nn.Linear(k, n, bias=True).to(torch.float16)
+    a = f8.Float8Linear.from_float(copy.deepcopy(lin), config=_cfg(f8, *scaling)).to(DEV)
+    b = f8.Float8Linear.from_float(copy.deepcopy(lin), config=_cfg(f8, *scaling)).to(DEV)
+    ref = copy.deepcopy(lin).to(DEV)
+    for it, mag in enumerate((1.0, 1e-6, 1.0)):   # the middle batch is tiny: 448 / amax would overflow fp16
+        x = (torch.randn(m, k) * mag).to(torch.float16).to(DEV)
+        dy = torch.randn(m, n).to(torch.float16).to(DEV)
+        outs = []
+        for mod, fwd in ((a, a.forward), (b, b.forward_composed)):
+            if "del" in scaling:
+                f8.sync_float8_amax_and_scale_history(mod)
+            xi = x.clone().requires_grad_()
+            mod.weight.grad = mod.bias.grad = None
+            y = fwd(xi)
+            y.backward(dy)
+            outs.append((y, xi.grad, mod.weight.grad))
+        for u, v in zip(*outs):
+            assert u.dtype == torch.float16 and torch.isfinite(u).all()
+            assert torch.equal(u, v), it
+        if scaling[0] == "dyn" and mag == 1.0:
+            assert to.sqnr(ref(x).detach().cpu(), outs[0][0].detach().cpu()) > 18.0
+    from float8_experimental_amd import _native
+
+    _, s = _native.amax_scale(torch.full((8, 8), 1e-7, dtype=torch.float16, device=DEV), torch.float8_e4m3fn)
+    assert s.item() == 65504.0
+
+
 @pytest.mark.parametrize("frozen", ["weight", "input"])
 def test_single_copy_path_with_one_gradient_not_needed(f8, frozen):
     torch.manual_seed(4)
