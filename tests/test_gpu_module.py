@@ -267,6 +267,29 @@ def test_fp16_layer_fused_equals_composed_and_scales_stay_finite(f8, scaling):
     assert s.item() == 65504.0
 
 
+def test_fused_equals_composed_over_a_random_sweep_of_sizes(f8):
+    """Whatever operand layouts and GEMM kernels the sizes select on the two routes (k-blocked or row-major; few-row,
+    128-row-tile, large-tile kernels; one fp8 copy or two), forward and both gradients are the same bits."""
+    rng = np.random.default_rng(7)
+    dims = [64, 100, 128, 200, 256, 320, 384, 448, 512, 640, 1024, 1152, 2048, 2304]
+    torch.manual_seed(13)
+    for case in range(24):
+        m, k, n = (int(rng.choice(dims)) for _ in range(3))
+        lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
+        a = f8.Float8Linear.from_float(copy.deepcopy(lin)).to(DEV)
+        b = f8.Float8Linear.from_float(copy.deepcopy(lin)).to(DEV)
+        x = torch.randn(m, k).to(torch.bfloat16).to(DEV)
+        dy = torch.randn(m, n).to(torch.bfloat16).to(DEV)
+        outs = []
+        for mod, fwd in ((a, a.forward), (b, b.forward_composed)):
+            xi = x.clone().requires_grad_()
+            y = fwd(xi)
+            y.backward(dy)
+            outs.append((y, xi.grad, mod.weight.grad))
+        for name, u, v in zip(("y", "dx", "dw"), *outs):
+            assert torch.equal(u, v), (case, m, k, n, name)
+
+
 @pytest.mark.parametrize("frozen", ["weight", "input"])
 def test_single_copy_path_with_one_gradient_not_needed(f8, frozen):
     torch.manual_seed(4)
