@@ -53,6 +53,22 @@ def test_host_side_argument_checks_need_no_gpu():
     assert rc == -1
     rc = lib.f8mi_sync(None, -1, 16, 0, 0, None)
     assert rc == -1
+    # k-blocked operands: k must be a multiple of 64 and at least 384 (unsupported, not invalid)
+    rc = lib.f8mi_gemm_nt_kb(None, 0, None, 0, i64(4), i64(4), i64(100), None, None, None, 0, i64(4), None, None)
+    assert rc == -2 and b"k-blocked" in lib.f8mi_last_error()
+    # transposed operands: (a transposed, bt not) is not built; row counts must be multiples of 64
+    rc = lib.f8mi_gemm_kb_ex(None, 0, 1, None, 0, 0, i64(64), i64(64), i64(384), None, None, None, 0, i64(64), None, None)
+    assert rc == -2
+    rc = lib.f8mi_gemm_kb_ex(None, 0, 0, None, 0, 1, i64(64), i64(100), i64(384), None, None, None, 0, i64(100), None, None)
+    assert rc == -2 and b"multiple of 64" in lib.f8mi_last_error()
+    rc = lib.f8mi_cast_layout(None, i64(4), i64(100), i64(100), 0, ctypes.c_void_p(8), 0, 0, ctypes.c_void_p(8), 1, None, 0, None, None)
+    assert rc == -2 and b"cols % 64" in lib.f8mi_last_error()
+    rc = lib.f8mi_cast_layout(None, i64(4), i64(64), i64(64), 0, ctypes.c_void_p(8), 0, 0, ctypes.c_void_p(8), 5, None, 0, None, None)
+    assert rc == -1
+    rc = lib.f8mi_cast_dynamic(None, i64(4), i64(4), i64(4), 0, 0, None, None, 0, None, 0, None, None)
+    assert rc == -1 and b"scale" in lib.f8mi_last_error()
+    rc = lib.f8mi_amax_scale_multi(None, 5000, i64(5000), 0, 0, 0, 0, ctypes.c_void_p(8), None, None, None)
+    assert rc == -1 and b"at most" in lib.f8mi_last_error()
 
 
 def test_cpu_tensors_are_refused_loudly():
