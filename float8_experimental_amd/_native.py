@@ -124,8 +124,14 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
         )
 
 
+def _raw_stream(dev: torch.device) -> int:
+    """hipStream_t of torch's current stream on ``dev`` as an integer (the raw accessor: no Stream object is built)."""
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(idx)
+
+
 def _stream(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return _raw_stream(t.device)
 
 
 _checked_devices = set()
@@ -147,7 +153,7 @@ _workspaces = {}
 def workspace(dev: torch.device) -> torch.Tensor:
     """Reduction workspace of f8mi_amax_scale (per-block partial maxima), one per (device, stream)."""
     _check_device(dev)
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _raw_stream(dev))
     ws = _workspaces.get(key)
     if ws is None:
         ws = torch.zeros(lib().f8mi_workspace_bytes() // 4, dtype=torch.int32, device=dev)
@@ -479,6 +485,6 @@ def probe_mfma(random_data: bool, iters: int = 4000, device: Optional[torch.devi
     out = C.c_double(0.0)
     with torch.cuda.device(dev):
         rc = lib().f8mi_probe_mfma(int(random_data), iters, scratch.data_ptr(), scratch.numel(), C.byref(out),
-                                   torch.cuda.current_stream(dev).cuda_stream)
+                                   _raw_stream(dev))
     _check(rc, "f8mi_probe_mfma")
     return out.value
