@@ -122,6 +122,11 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
             f"{name} is on {t.device}: float8_experimental_amd computes on MI355X device tensors only "
             "(no CPU fallback)"
         )
+    if t.device.index is not None and t.device.index != torch.cuda.current_device():
+        # the library launches on the tensor's stream with whatever device is current: one process per GPU, or
+        # `with torch.cuda.device(t.device):` around the call, keeps the two the same
+        raise Float8NativeError(f"{name} is on {t.device} but the current device is cuda:{torch.cuda.current_device()}: "
+                                "make the tensor's device current (torch.cuda.set_device / torch.cuda.device)")
 
 
 def _raw_stream(dev: torch.device) -> int:
