@@ -62,7 +62,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_kernel(
     // ---- which tile
     int lid = blockIdx.x;
     const int npid = gridDim.x;
-    if (npid % NUM_XCD == 0) lid = (lid % NUM_XCD) * (npid / NUM_XCD) + lid / NUM_XCD;
+    lid = xcd_contiguous_id(lid, npid);
     const int width = GROUP_M * tiles_n;
     const int group = lid / width;
     const int first_m = group * GROUP_M;

@@ -159,7 +159,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
     // ---- which tile (same walk as the other kernels)
     int lid = blockIdx.x;
     const int npid = gridDim.x;
-    if (npid % NUM_XCD == 0) lid = (lid % NUM_XCD) * (npid / NUM_XCD) + lid / NUM_XCD;
+    lid = xcd_contiguous_id(lid, npid);
     // The walk sweeps along the longer side of the tile grid in bands GROUP tiles wide, so that an XCD's 32
     // workgroups hold a 4 x 8 (or 8 x 4) patch of neighbouring tiles; sweeping along the shorter side instead
     // cost 1 - 3 % on the shapes where the sides differ most (measured both ways on all twelve benchmark GEMMs).

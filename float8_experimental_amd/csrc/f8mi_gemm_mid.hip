@@ -51,7 +51,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
     // consecutive workgroup ids go to the 8 XCDs round-robin; re-deal them so that one XCD (one L2) gets a
     // contiguous run of the tile order (rows fastest): the workgroups that share a block of Bt sit behind the same L2
     int lid = blockIdx.x;
-    if (gridDim.x % NUM_XCD == 0) lid = (lid % NUM_XCD) * (gridDim.x / NUM_XCD) + lid / NUM_XCD;
+    lid = xcd_contiguous_id(lid, gridDim.x);
     const int tm = lid % tiles_m, tn = lid / tiles_m;
     const int m0 = tm * MID_TILE_M, n0 = tn * Cfg::TILE_N;
     const int lane = threadIdx.x & 63;

@@ -21,6 +21,13 @@ constexpr int GROUP_M = 8;
 constexpr int NUM_XCD = 8;
 constexpr int MID_MAX_TILES_256 = 64;
 
+// Consecutive workgroup ids go to the 8 XCDs round-robin.  Re-deals them so that XCD x (ids x, x+8, ...) works on
+// a contiguous run of the tile order -- whatever the grid size: the first `grid % 8` XCDs get one workgroup more.
+__device__ __forceinline__ int xcd_contiguous_id(int bid, int grid) {
+    const int x = bid % NUM_XCD, q = grid / NUM_XCD, r = grid % NUM_XCD;
+    return x * q + min(x, r) + bid / NUM_XCD;
+}
+
 #define F8MI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 // Workgroup barrier that waits for this wave's LDS traffic only.
