@@ -204,6 +204,15 @@ def test_fsdp_flag_and_precompute_on_the_host():
         f8.precompute_float8_dynamic_scale_for_fsdp(nn.Sequential(lin))
 
 
+def test_tensor_parallel_styles_say_that_they_need_several_gpus():
+    from float8_experimental_amd.float8_tensor_parallel import (Float8ColwiseParallel, Float8RowwiseParallel,
+                                                                PrepareFloat8ModuleInput)
+
+    for style in (Float8ColwiseParallel, Float8RowwiseParallel, PrepareFloat8ModuleInput):
+        with pytest.raises(NotImplementedError, match="single MI355X"):
+            style()
+
+
 def test_float8_tensor_metadata_on_cpu():
     data = torch.zeros(4, 8, dtype=torch.float8_e4m3fn)
     t = Float8Tensor(data, torch.tensor(2.0), torch.bfloat16, None)
