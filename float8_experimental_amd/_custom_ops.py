@@ -1,13 +1,19 @@
-"""The fused dynamic-scaling linear as two ``torch.library`` custom ops, so that ``torch.compile`` sees
-one opaque node per direction instead of tracing into the ctypes calls (which it cannot).
+"""The fused linear as two ``torch.library`` custom ops, so that ``torch.compile`` sees one opaque node per
+direction instead of tracing into the ctypes calls (which it cannot).
 
 The reference keeps its float8 pieces traceable with ``torch._dynamo.allow_in_graph``
 (float8_linear.py:43, float8_tensor.py:131,198) and lets inductor generate the casts; here the kernels
-are hand-written, so the compiler only has to know shapes and dtypes (the fake implementations below)
-and how gradients flow (``register_autograd``).  Modules with delayed scaling keep state on the module
-(flags, amax / scale buffers) and are run outside the graph instead (``torch._dynamo.disable``).
+are hand-written, so the compiler only has to know shapes and dtypes (the fake implementations below) and how
+gradients flow (``register_autograd``).  Each of the three tensors is scaled dynamically (no buffers passed)
+or with the delayed-scaling buffers of the module: the cast then uses the existing scale and records this
+step's amax.  The ops are functional (an op that writes its arguments cannot carry an autograd formula): they
+return the new amax as a one-element tensor and the caller copies it into the module's buffer, an in-place
+update of a buffer that the compiler knows how to trace.
+What stays outside the graph (``torch._dynamo.disable`` on the module) is everything that keeps *Python* state:
+the first-iteration amax initialisation and the pre/post-forward flags -- configure
+``enable_amax_init=False, enable_pre_and_post_forward=False`` for a graph without breaks, as with the reference.
 """
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 
@@ -22,94 +28,134 @@ def _layout(t_rows: int, t_cols: int, kblock: bool):
     return (t_cols // _KB, t_rows, _KB) if kblock else (t_rows, t_cols)
 
 
-def _cast_dynamic(t2d, float8_dtype, want_row, want_t, row_kb, t_kb):
-    return _native.cast_dynamic(t2d, float8_dtype, want_out=want_row, want_out_t=want_t, out_kblock=row_kb, out_t_kblock=t_kb)
+def _cast(t2d, float8_dtype, scale_buf, want_row, want_t, row_kb, t_kb):
+    """(row copy, transposed copy, scale used, new amax): dynamic scaling without a scale buffer (new amax: empty),
+    else the delayed-scaling cast (existing scale, fp32 product, this step's amax in a fresh one-element tensor;
+    float8_scaling_utils.py:65-96)."""
+    if scale_buf is None:
+        row, tr, scale = _native.cast_dynamic(t2d, float8_dtype, want_out=want_row, want_out_t=want_t, out_kblock=row_kb,
+                                              out_t_kblock=t_kb)
+        return row, tr, scale, torch.empty(0, dtype=torch.float32, device=t2d.device)
+    amax = torch.empty(1, dtype=torch.float32, device=t2d.device)
+    row, tr = _native.cast(t2d, scale_buf, float8_dtype, product_dtype=torch.float32, want_out=want_row, want_out_t=want_t,
+                           amax_out=amax, out_kblock=row_kb, out_t_kblock=t_kb)
+    return row, tr, scale_buf, amax
 
 
 def _gemm(a8, sa, b8, sb, out_dtype, kb):
     return _native.gemm_nt_kb(a8, sa, b8, sb, out_dtype) if kb else _native.gemm_nt(a8, sa, b8, sb, out_dtype)
 
 
-@torch.library.custom_op("f8mi::linear_dynamic_fwd", mutates_args=())
-def linear_dynamic_fwd(x2: torch.Tensor, weight: torch.Tensor, need_dx: bool, need_dw: bool) -> Tuple[
-        torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    """y = x2 W^T in fp8 with dynamic scales; also the fp8 copies and scales backward needs.
+@torch.library.custom_op("f8mi::linear_fwd", mutates_args=())
+def linear_fwd(x2: torch.Tensor, weight: torch.Tensor, need_dx: bool, need_dw: bool,
+               scale_x: Optional[torch.Tensor], scale_w: Optional[torch.Tensor]) -> Tuple[
+        torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """y = x2 W^T in fp8; also the fp8 copies and the dynamic scales backward needs, and the amaxes delayed scaling records.
 
-    Returns (y, xs, ws, sx, sw).  When every dimension allows it (``_native.tn_ok``) xs / ws are the forward's
-    own k-blocked operands (backward reads them transposed); otherwise they are the transposed copies, and
-    one that backward will not need is an empty tensor."""
+    Returns (y, xs, ws, sx, sw, amax_x, amax_w).  When the sizes allow it (``_native.tn_ok``) xs / ws are the
+    forward's own k-blocked operands (backward reads them transposed); otherwise they are the transposed copies,
+    and one that backward will not need is an empty tensor.  sx / sw are the scales of dynamically scaled
+    tensors; for a tensor with delayed scaling (``scale_*`` given: the module's scale buffer) the slot holds an empty
+    tensor and ``amax_*`` this step's amax, [1] fp32 (empty for dynamic scaling)."""
     m, k = x2.shape
     n = weight.shape[0]
+    none = lambda dt: torch.empty(0, dtype=dt, device=x2.device)
+    out_s = lambda s, buf: s if buf is None else none(torch.float32)
     if _native.tn_ok(m, k, n):
-        x8, _, sx = _cast_dynamic(x2, e4m3_dtype, True, False, True, False)
-        w8, _, sw = _cast_dynamic(weight, e4m3_dtype, True, False, True, False)
-        return _native.gemm_nt_kb(x8, sx, w8, sw, x2.dtype), x8, w8, sx, sw
+        x8, _, sx, ax = _cast(x2, e4m3_dtype, scale_x, True, False, True, False)
+        w8, _, sw, aw = _cast(weight, e4m3_dtype, scale_w, True, False, True, False)
+        return _native.gemm_nt_kb(x8, sx, w8, sw, x2.dtype), x8, w8, out_s(sx, scale_x), out_s(sw, scale_w), ax, aw
     kb_fwd, kb_dx, kb_dw = _native.kblock_ok(k), _native.kblock_ok(n), _native.kblock_ok(m)
-    x8, x8t, sx = _cast_dynamic(x2, e4m3_dtype, True, need_dw, kb_fwd, kb_dw)
-    w8, w8t, sw = _cast_dynamic(weight, e4m3_dtype, True, need_dx, kb_fwd, kb_dx)
+    x8, x8t, sx, ax = _cast(x2, e4m3_dtype, scale_x, True, need_dw, kb_fwd, kb_dw)
+    w8, w8t, sw, aw = _cast(weight, e4m3_dtype, scale_w, True, need_dx, kb_fwd, kb_dx)
     y = _gemm(x8, sx, w8, sw, x2.dtype, kb_fwd)
-    empty = lambda: torch.empty(0, dtype=e4m3_dtype, device=x2.device)
-    return y, (x8t if need_dw else empty()), (w8t if need_dx else empty()), sx, sw
+    return (y, (x8t if need_dw else none(e4m3_dtype)), (w8t if need_dx else none(e4m3_dtype)),
+            out_s(sx, scale_x), out_s(sw, scale_w), ax, aw)
 
 
-@linear_dynamic_fwd.register_fake
-def _(x2, weight, need_dx, need_dw):
+@linear_fwd.register_fake
+def _(x2, weight, need_dx, need_dw, scale_x, scale_w):
     m, k = x2.shape
     n = weight.shape[0]
     f8 = lambda shape: torch.empty(shape, dtype=e4m3_dtype, device=x2.device)
-    s = lambda: torch.empty((), dtype=torch.float32, device=x2.device)
+    s = lambda buf: torch.empty(() if buf is None else (0,), dtype=torch.float32, device=x2.device)
+    a = lambda buf: torch.empty((0,) if buf is None else (1,), dtype=torch.float32, device=x2.device)
     y = torch.empty((m, n), dtype=x2.dtype, device=x2.device)
     if _native.tn_ok(m, k, n):
-        return y, f8((k // _KB, m, _KB)), f8((k // _KB, n, _KB)), s(), s()
+        return y, f8((k // _KB, m, _KB)), f8((k // _KB, n, _KB)), s(scale_x), s(scale_w), a(scale_x), a(scale_w)
     kb_dx, kb_dw = _native.kblock_ok(n), _native.kblock_ok(m)
-    return (y, f8(_layout(k, m, kb_dw)) if need_dw else f8((0,)), f8(_layout(k, n, kb_dx)) if need_dx else f8((0,)), s(), s())
+    return (y, f8(_layout(k, m, kb_dw)) if need_dw else f8((0,)), f8(_layout(k, n, kb_dx)) if need_dx else f8((0,)),
+            s(scale_x), s(scale_w), a(scale_x), a(scale_w))
 
 
-@torch.library.custom_op("f8mi::linear_dynamic_bwd", mutates_args=())
-def linear_dynamic_bwd(dy2: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor,
-                       k: int, need_dx: bool, need_dw: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(dx, dw) = (dY W, dY^T x) in fp8, dY cast to e5m2 with a dynamic scale; an unneeded one is empty."""
+@torch.library.custom_op("f8mi::linear_bwd", mutates_args=())
+def linear_bwd(dy2: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor,
+               k: int, need_dx: bool, need_dw: bool, scale_g: Optional[torch.Tensor]) -> Tuple[
+        torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dx, dw, amax_g): (dY W, dY^T x) in fp8, dY cast to e5m2 with a dynamic scale or the delayed-scaling scale
+    buffer (then amax_g is this step's amax of dY, [1] fp32; else empty); an unneeded gradient is empty."""
     m, n = dy2.shape
     empty = lambda: torch.empty(0, dtype=dy2.dtype, device=dy2.device)
     if _native.tn_ok(m, k, n):
-        g8, _, sg = _cast_dynamic(dy2, e5m2_dtype, True, False, True, False)
+        g8, _, sg, ag = _cast(dy2, e5m2_dtype, scale_g, True, False, True, False)
         dx = _native.gemm_kb_ex(g8, False, sg, ws, True, sw, dy2.dtype) if need_dx else empty()
         dw = _native.gemm_kb_ex(g8, True, sg, xs, True, sx, dy2.dtype) if need_dw else empty()
-        return dx, dw
+        return dx, dw, ag
     kb_dx, kb_dw = _native.kblock_ok(n), _native.kblock_ok(m)
-    g8, g8t, sg = _cast_dynamic(dy2, e5m2_dtype, need_dx, need_dw, kb_dx, kb_dw)
+    g8, g8t, sg, ag = _cast(dy2, e5m2_dtype, scale_g, need_dx, need_dw, kb_dx, kb_dw)
     dx = _gemm(g8, sg, ws, sw, dy2.dtype, kb_dx) if need_dx else empty()
     dw = _gemm(g8t, sg, xs, sx, dy2.dtype, kb_dw) if need_dw else empty()
-    return dx, dw
+    return dx, dw, ag
 
 
-@linear_dynamic_bwd.register_fake
-def _(dy2, xs, ws, sx, sw, k, need_dx, need_dw):
+@linear_bwd.register_fake
+def _(dy2, xs, ws, sx, sw, k, need_dx, need_dw, scale_g):
     m, n = dy2.shape
     e = lambda shape: torch.empty(shape, dtype=dy2.dtype, device=dy2.device)
-    return (e((m, k)) if need_dx else e((0,)), e((n, k)) if need_dw else e((0,)))
+    return (e((m, k)) if need_dx else e((0,)), e((n, k)) if need_dw else e((0,)),
+            torch.empty((0,) if scale_g is None else (1,), dtype=torch.float32, device=dy2.device))
 
 
-def _setup_context(ctx, inputs, output):
-    x2, weight, need_dx, need_dw = inputs
-    _, x8t, w8t, sx, sw = output
-    ctx.k = x2.shape[1]
-    ctx.need = (need_dx, need_dw)
-    ctx.save_for_backward(x8t, w8t, sx, sw)
+class _LinearFn(torch.autograd.Function):
+    """Autograd around the two functional ops; the amax buffers of delayed scaling are updated in place here, where
+    the compiler traces ordinary tensor operations."""
+
+    @staticmethod
+    def forward(ctx, x2, weight, bufs_x, bufs_w, bufs_g):
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        sx_buf = bufs_x[1] if bufs_x is not None else None
+        sw_buf = bufs_w[1] if bufs_w is not None else None
+        y, xs, ws, sx, sw, ax, aw = linear_fwd(x2, weight, need_dx, need_dw, sx_buf, sw_buf)
+        if bufs_x is not None:
+            bufs_x[0].copy_(ax)
+        if bufs_w is not None:
+            bufs_w[0].copy_(aw)
+        ctx.k = x2.shape[1]
+        ctx.bufs_g = bufs_g
+        # a delayed tensor's scale is the module's buffer, a dynamic one's comes out of the forward op
+        ctx.save_for_backward(xs, ws, sx if sx_buf is None else sx_buf, sw if sw_buf is None else sw_buf)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        xs, ws, sx, sw = ctx.saved_tensors
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        bufs_g = ctx.bufs_g
+        dx, dw, ag = linear_bwd(gy.contiguous(), xs, ws, sx, sw, ctx.k, need_dx, need_dw,
+                                bufs_g[1] if bufs_g is not None else None)
+        if bufs_g is not None:
+            bufs_g[0].copy_(ag)
+        return (dx if need_dx else None), (dw if need_dw else None), None, None, None
 
 
-def _backward(ctx, gy, *_unused):
-    x8t, w8t, sx, sw = ctx.saved_tensors
-    need_dx, need_dw = ctx.need
-    dx, dw = linear_dynamic_bwd(gy.contiguous(), x8t, w8t, sx, sw, ctx.k, need_dx, need_dw)
-    return (dx if need_dx else None), (dw if need_dw else None), None, None
-
-
-linear_dynamic_fwd.register_autograd(_backward, setup_context=_setup_context)
+def linear(x: torch.Tensor, weight: torch.Tensor, bufs_x=None, bufs_w=None, bufs_g=None) -> torch.Tensor:
+    """y = x W^T with fp8 matmuls in both directions, traceable by ``torch.compile`` as one node per direction.
+    ``bufs_*``: (amax, scale) buffers of a tensor with delayed scaling, None for dynamic scaling."""
+    k = x.shape[-1]
+    y = _LinearFn.apply(x.reshape(-1, k), weight, bufs_x, bufs_w, bufs_g)
+    return y.reshape(*x.shape[:-1], weight.shape[0])
 
 
 def linear_dynamic(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """y = x W^T, all three tensors dynamically scaled; traceable by ``torch.compile`` as one node."""
-    k = x.shape[-1]
-    y = linear_dynamic_fwd(x.reshape(-1, k), weight, x.requires_grad, weight.requires_grad)[0]
-    return y.reshape(*x.shape[:-1], weight.shape[0])
+    """``linear`` with all three tensors dynamically scaled."""
+    return linear(x, weight)

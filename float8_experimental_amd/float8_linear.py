@@ -330,15 +330,24 @@ class Float8Linear(torch.nn.Linear):
         return self._forward_eager(input)
 
     def _forward_under_compile(self, input: torch.Tensor) -> torch.Tensor:
-        """What ``torch.compile`` traces: all-dynamic scaling is one custom-op node (plus the bias add);
-        anything that keeps state on the module, or carries Float8Tensors, runs outside the graph."""
-        plain = (not self.has_any_delayed_scaling and not self.config.emulate and self._precomputed_weight_scale is None
+        """What ``torch.compile`` traces: one custom-op node per direction (plus the bias add), with the delayed-scaling
+        buffers as arguments the node writes.  Anything that keeps Python state -- the first-iteration amax
+        initialisation, the pre/post-forward flags (``enable_amax_init`` / ``enable_pre_and_post_forward``: switch both
+        off for a graph without breaks, as with the reference) -- or carries Float8Tensors runs outside the graph."""
+        stateless = (not self.has_any_delayed_scaling
+                     or (self.is_amax_initialized and not self.enable_pre_and_post_forward))
+        plain = (stateless and not self.config.emulate and self._precomputed_weight_scale is None
                  and not isinstance(self.weight, Float8Tensor) and not isinstance(input, Float8Tensor))
         if not plain:
             return self._forward_outside_graph(input)
-        from ._custom_ops import linear_dynamic
+        from ._custom_ops import linear
 
-        output = linear_dynamic(self._autocast_input(input), self.weight)
+        def bufs(kind):
+            if getattr(self, f"scaling_type_{kind}") is not ScalingType.DELAYED:
+                return None
+            return getattr(self, f"fp8_amax_{kind}"), getattr(self, f"fp8_scale_{kind}")
+
+        output = linear(self._autocast_input(input), self.weight, bufs("input"), bufs("weight"), bufs("grad_output"))
         if self.bias is not None:
             output = output + self.bias.to(output.dtype)
         return output

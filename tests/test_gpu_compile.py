@@ -72,6 +72,35 @@ def test_frozen_weight_and_no_grad_under_compile(f8):
 
 
 @pytest.mark.parametrize("backend", ["eager", "aot_eager"])
+@pytest.mark.parametrize("kinds", ["DDD", "DyD", "yDy"])  # input, weight, grad_output: D delayed, y dynamic
+@pytest.mark.parametrize("shape,n", [((32, 512), 448), ((3, 768, 2048), 2432)])
+def test_delayed_scaling_compiles_as_one_graph(f8, backend, kinds, shape, n):
+    """Reference: test_compile.py runs delayed scaling with enable_amax_init=False, enable_pre_and_post_forward=False
+    under fullgraph=True.  Here the amax buffers are written by the graph; the sync stays an eager call between steps."""
+    torch.manual_seed(4)
+    st = lambda c: f8.CastConfig(f8.ScalingType.DELAYED if c == "D" else f8.ScalingType.DYNAMIC)
+    cfg = f8.Float8LinearConfig(cast_config_input=st(kinds[0]), cast_config_weight=st(kinds[1]),
+                                cast_config_grad_output=st(kinds[2]), enable_amax_init=False,
+                                enable_pre_and_post_forward=False)
+    k = shape[-1]
+    base = nn.Sequential(nn.Linear(k, n, bias=True), nn.GELU(), nn.Linear(n, 384, bias=False)).to(DEV, dtype=torch.bfloat16)
+    a, b = copy.deepcopy(base), copy.deepcopy(base)
+    f8.convert_to_float8_training(a, config=cfg)
+    f8.convert_to_float8_training(b, config=cfg)
+    torch._dynamo.reset()
+    cb = torch.compile(b, backend=backend, fullgraph=True)
+    for it in range(4):
+        x = torch.randn(shape, device=DEV, dtype=torch.bfloat16) * 1.5 ** it
+        dy = torch.randn(*shape[:-1], 384, device=DEV, dtype=torch.bfloat16) * 10.0 ** (it - 2)
+        f8.sync_float8_amax_and_scale_history(a)
+        f8.sync_float8_amax_and_scale_history(b)
+        for u, v in zip(_run(cb, x, dy), _run(a, x, dy)):
+            assert torch.equal(u, v), it
+        for (name, b1), (_, b2) in zip(a.named_buffers(), b.named_buffers()):
+            assert torch.equal(b1, b2), (it, name)
+
+
+@pytest.mark.parametrize("backend", ["eager", "aot_eager"])
 def test_delayed_scaling_and_inference_modules_run_outside_the_graph(f8, backend):
     """State-carrying modules are not traced (graph break); compiled and eager runs still agree exactly."""
     from float8_experimental_amd.inference import ActivationCasting, QuantConfig, quantize_to_float8
