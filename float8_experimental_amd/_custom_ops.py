@@ -13,7 +13,7 @@ What stays outside the graph (``torch._dynamo.disable`` on the module) is everyt
 the first-iteration amax initialisation and the pre/post-forward flags -- configure
 ``enable_amax_init=False, enable_pre_and_post_forward=False`` for a graph without breaks, as with the reference.
 """
-from typing import Optional, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -159,3 +159,27 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bufs_x=None, bufs_w=None, bufs
 def linear_dynamic(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``linear`` with all three tensors dynamically scaled."""
     return linear(x, weight)
+
+
+_sync_tables = {}
+
+
+@torch.library.custom_op("f8mi::sync", mutates_args=("scales",))
+def sync(amaxes: List[torch.Tensor], histories: List[torch.Tensor], scales: List[torch.Tensor], is_e5m2: List[bool],
+         orig_is_fp16: bool) -> None:
+    """The delayed-scaling sync of all listed buffers as one node (and one kernel launch): for each i,
+    ``scales[i] = fmax / max(amaxes[i], histories[i][:-1])`` in the reference's rounding
+    (float8_linear_utils.py:287-319).  No autograd: the buffers carry none."""
+    key = tuple(t.data_ptr() for group in (amaxes, histories, scales) for t in group)
+    table = _sync_tables.get(key)
+    if table is None:
+        if len(_sync_tables) > 64:
+            _sync_tables.clear()
+        rows = [(a, h, s, e5m2_dtype if e else e4m3_dtype) for a, h, s, e in zip(amaxes, histories, scales, is_e5m2)]
+        table = _sync_tables[key] = _native.sync_table(rows, amaxes[0].device)
+    _native.sync(table, histories[0].numel(), orig_is_fp16, writeback_history=False)
+
+
+@sync.register_fake
+def _(amaxes, histories, scales, is_e5m2, orig_is_fp16):
+    return None

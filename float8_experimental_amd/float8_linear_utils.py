@@ -120,8 +120,19 @@ def sync_float8_amax_and_scale_history(model: torch.nn.Module, fp8_layers=None) 
     if torch.distributed.is_available() and torch.distributed.is_initialized() and torch.distributed.get_world_size() > 1:
         raise NotImplementedError("amax all-reduce across ranks: this build drives a single GPU")
 
-    table = _sync_table(fp8_layers)
-    _native.sync(table, next(iter(hist_lens)), next(iter(x_dtypes)) is torch.float16, writeback_history=False)
+    orig_is_fp16 = next(iter(x_dtypes)) is torch.float16
+    if torch.compiler.is_compiling():
+        # the same launch as one opaque node that writes the scale buffers (reference: test_compile.py:257-274
+        # compiles this function into a single frame)
+        from ._custom_ops import sync
+
+        rows = [(child, kind, f8) for child in fp8_layers for kind, f8 in _KINDS]
+        sync([getattr(c, f"fp8_amax_{kind}") for c, kind, _ in rows],
+             [getattr(c, f"fp8_amax_history_{kind}") for c, kind, _ in rows],
+             [getattr(c, f"fp8_scale_{kind}") for c, kind, _ in rows],
+             [f8 is e5m2_dtype for _, _, f8 in rows], orig_is_fp16)
+    else:
+        _native.sync(_sync_table(fp8_layers), next(iter(hist_lens)), orig_is_fp16, writeback_history=False)
 
     for child in fp8_layers:
         child.amax_and_scale_synced = True

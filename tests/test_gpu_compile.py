@@ -100,6 +100,73 @@ def test_delayed_scaling_compiles_as_one_graph(f8, backend, kinds, shape, n):
             assert torch.equal(b1, b2), (it, name)
 
 
+@pytest.mark.parametrize("backend", ["eager", "aot_eager", "inductor"])
+def test_sync_compiles_into_one_frame(f8, backend):
+    """Reference: test_compile.py:257-274 (one frame) and :294-320 (fullgraph): the sync of all layers is one node."""
+    from torch._dynamo.testing import CompileCounterWithBackend
+
+    torch.manual_seed(5)
+    D = f8.CastConfig(f8.ScalingType.DELAYED)
+    cfg = f8.Float8LinearConfig(cast_config_input=D, cast_config_weight=D, cast_config_grad_output=D)
+    base = nn.Sequential(nn.Linear(256, 320, bias=True), nn.ReLU(), nn.Linear(320, 128, bias=True)).to(DEV, dtype=torch.bfloat16)
+    a, b = copy.deepcopy(base), copy.deepcopy(base)
+    f8.convert_to_float8_training(a, config=cfg)
+    f8.convert_to_float8_training(b, config=cfg)
+    torch._dynamo.reset()
+    cnts = CompileCounterWithBackend(backend)
+    csync = torch.compile(f8.sync_float8_amax_and_scale_history, backend=cnts, fullgraph=True)
+    for it in range(3):
+        x = torch.randn(48, 256, device=DEV, dtype=torch.bfloat16) * 3.0 ** it
+        dy = torch.randn(48, 128, device=DEV, dtype=torch.bfloat16)
+        f8.sync_float8_amax_and_scale_history(a)
+        try:
+            csync(b)
+        except Exception as e:
+            if backend == "inductor" and it == 0:
+                pytest.skip(f"inductor cannot generate code here: {type(e).__name__}")
+            raise
+        if it == 0:
+            assert cnts.frame_count == 1
+        for (name, b1), (_, b2) in zip(a.named_buffers(), b.named_buffers()):
+            assert torch.equal(b1, b2), (it, name)
+        for u, v in zip(_run(b, x, dy), _run(a, x, dy)):
+            assert torch.equal(u, v), it
+    # one more specialisation once the layers have seen an input (their recorded input dtype goes from None to bf16)
+    assert cnts.frame_count == 2
+    assert all(m.amax_and_scale_synced is False for m in f8.float8_linear_utils.get_float8_layers(b))  # post-forward ran
+
+
+def test_whole_delayed_scaling_step_as_one_graph(f8):
+    """sync + forward in one compiled function: the scales the sync node writes are the ones the casts read."""
+    torch.manual_seed(6)
+    D = f8.CastConfig(f8.ScalingType.DELAYED)
+    cfg = f8.Float8LinearConfig(cast_config_input=D, cast_config_weight=D, cast_config_grad_output=D,
+                                enable_amax_init=False, enable_pre_and_post_forward=False)
+    base = nn.Sequential(nn.Linear(512, 640, bias=False), nn.GELU(), nn.Linear(640, 384, bias=True)).to(DEV, dtype=torch.bfloat16)
+    a, b = copy.deepcopy(base), copy.deepcopy(base)
+    f8.convert_to_float8_training(a, config=cfg)
+    f8.convert_to_float8_training(b, config=cfg)
+
+    def step(mod, x):
+        f8.sync_float8_amax_and_scale_history(mod)
+        return mod(x)
+
+    torch._dynamo.reset()
+    cstep = torch.compile(step, backend="aot_eager", fullgraph=True)
+    for it in range(4):
+        x = torch.randn(96, 512, device=DEV, dtype=torch.bfloat16) * 2.0 ** it
+        dy = torch.randn(96, 384, device=DEV, dtype=torch.bfloat16) * 0.1 ** it
+        xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+        ya, yb = step(a, xa), cstep(b, xb)
+        ya.backward(dy)
+        yb.backward(dy)
+        assert torch.equal(ya, yb) and torch.equal(xa.grad, xb.grad), it
+        for pa, pb in zip(a.parameters(), b.parameters()):
+            assert torch.equal(pa.grad, pb.grad), it
+        for (name, b1), (_, b2) in zip(a.named_buffers(), b.named_buffers()):
+            assert torch.equal(b1, b2), (it, name)
+
+
 @pytest.mark.parametrize("backend", ["eager", "aot_eager"])
 def test_delayed_scaling_and_inference_modules_run_outside_the_graph(f8, backend):
     """State-carrying modules are not traced (graph break); compiled and eager runs still agree exactly."""
