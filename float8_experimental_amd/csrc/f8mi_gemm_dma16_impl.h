@@ -39,13 +39,11 @@ __device__ __forceinline__ void mfma16_first(v4f& acc, const v8i& first, const v
 // acc[tj][ti] as left by MFMA(first = Bt rows, second = A rows): lane holds row ti*16 + lane%16
 // and the four columns tj*16 + 4*(lane/16) + e of its wave's 128 x 128 quarter.
 template <int C_DT>
-__device__ __forceinline__ void store_c_tile16(v4f (&acc)[8][8], uint8_t* smem, int m0, int n0, int M, int N,
-                                               const float* __restrict__ sa_dev, const float* __restrict__ sb_dev,
+__device__ __forceinline__ void store_c_tile16(v4f (&acc)[8][8], int m0, int n0, int M, int N, float inv,
                                                void* __restrict__ C, int64_t ldc, const void* __restrict__ bias,
                                                int c_vec_ok) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
     const int lm = lane & 15, lq = lane >> 4;
     const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
 
@@ -78,44 +76,46 @@ __device__ __forceinline__ void store_c_tile16(v4f (&acc)[8][8], uint8_t* smem, 
             }
         }
     } else {
-        lds_barrier();  // all waves are done with the operand slabs before they become the output staging area
-        uint8_t* ep = smem + wave * (128 * EPI_PITCH);
+        // 16-bit outputs straight from the registers.  A lane holds 4 neighbouring columns of a row (8 bytes) of
+        // each accumulator tile; v_permlane16_swap between the tiles tj = 2p and 2p + 1 trades the odd 16-lane rows
+        // of the first for the even ones of the second, after which every lane holds 8 neighbouring columns
+        // (lq even: columns 4 lq .. 4 lq + 7 of tile 2p; lq odd: columns 4 (lq - 1) .. + 7 of tile 2p + 1) and one
+        // 16-byte store per lane writes 64 contiguous bytes of 16 rows.  (Staging the tile through LDS for 256-byte
+        // row segments took twice the time: with one wave per SIMD nothing hides the round trip.)
+        uint16_t* Ch = (uint16_t*)C;
+        float bv[8][4];
 #pragma unroll
         for (int tj = 0; tj < 8; tj++) {
-            const int cl = tj * 16 + 4 * lq;  // column inside the wave's 128
-            float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (bias) {
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (wcol0 + cl + r < N) bv[r] = load_bias<C_DT>(bias, wcol0 + cl + r);
-            }
-#pragma unroll
-            for (int ti = 0; ti < 8; ti++) {
-                const float v0 = acc[tj][ti][0] * inv + bv[0];
-                const float v1 = acc[tj][ti][1] * inv + bv[1];
-                const float v2 = acc[tj][ti][2] * inv + bv[2];
-                const float v3 = acc[tj][ti][3] * inv + bv[3];
-                *(uint2*)(ep + (ti * 16 + lm) * EPI_PITCH + cl * 2) = make_uint2(pack2<C_DT>(v0, v1), pack2<C_DT>(v2, v3));
+            for (int r = 0; r < 4; r++) {
+                const int col = wcol0 + tj * 16 + 4 * lq + r;
+                bv[tj][r] = (bias && col < N) ? load_bias<C_DT>(bias, col) : 0.f;
             }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own wave's tile only: no workgroup barrier needed
-        uint16_t* Ch = (uint16_t*)C;
-        const int chunk = lane & 15, rsub = lane >> 4;
-        const int col = wcol0 + chunk * 8;
-#pragma unroll 4
-        for (int it = 0; it < 32; it++) {
-            const int rl = it * 4 + rsub;
-            const int row = wrow0 + rl;
-            const uint4 v = *(const uint4*)(ep + rl * EPI_PITCH + chunk * 16);
-            if (row < M && col < N) {
-                uint16_t* dst = Ch + (int64_t)row * ldc + col;
-                if (c_vec_ok && col + 8 <= N) {
-                    *(uint4*)dst = v;
-                } else {
-                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const int col_l = (lq & 1) * 16 + (lq >> 1) * 8;  // inside the 32 columns of a pair of tiles
 #pragma unroll
-                    for (int i = 0; i < 8; i++)
-                        if (col + i < N) dst[i] = (uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+        for (int ti = 0; ti < 8; ti++) {
+            const int row = wrow0 + ti * 16 + lm;
+#pragma unroll
+            for (int tp = 0; tp < 4; tp++) {
+                const int te = 2 * tp, to = 2 * tp + 1;
+                const uint32_t x0 = pack2<C_DT>(acc[te][ti][0] * inv + bv[te][0], acc[te][ti][1] * inv + bv[te][1]);
+                const uint32_t x1 = pack2<C_DT>(acc[te][ti][2] * inv + bv[te][2], acc[te][ti][3] * inv + bv[te][3]);
+                const uint32_t y0 = pack2<C_DT>(acc[to][ti][0] * inv + bv[to][0], acc[to][ti][1] * inv + bv[to][1]);
+                const uint32_t y1 = pack2<C_DT>(acc[to][ti][2] * inv + bv[to][2], acc[to][ti][3] * inv + bv[to][3]);
+                const auto s0 = __builtin_amdgcn_permlane16_swap(x0, y0, false, false);  // all lanes take part
+                const auto s1 = __builtin_amdgcn_permlane16_swap(x1, y1, false, false);
+                const int col = wcol0 + tp * 32 + col_l;
+                if (row < M && col < N) {
+                    uint16_t* dst = Ch + (int64_t)row * ldc + col;
+                    if (c_vec_ok && col + 8 <= N) {
+                        *(uint4*)dst = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                    } else {
+                        const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
+#pragma unroll
+                        for (int i = 0; i < 8; i++)
+                            if (col + i < N) dst[i] = (uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+                    }
                 }
             }
         }
@@ -179,6 +179,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
         tn = (lid % width) / gsz;
     }
     const int m0 = tm * BM, n0 = tn * BN;
+    // 1 / (sa * sb) for the epilogue, fetched now and kept in a scalar register: loaded after the main loop, the two
+    // scales were a memory round trip with nothing to hide it
+    const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
+        int, __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev))));
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -388,7 +392,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
     // the last MFMAs are still in the pipeline (8 passes): keep the accumulator reads away from them
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
-    store_c_tile16<C_DT>(acc, smem, m0, n0, M, N, sa_dev, sb_dev, C, ldc, bias, c_vec_ok);
+    store_c_tile16<C_DT>(acc, m0, n0, M, N, inv, C, ldc, bias, c_vec_ok);
 }
 
 template <int AF, int BF, int C_DT, bool ODD, bool A_TR, bool B_TR>
