@@ -35,55 +35,46 @@ __device__ __forceinline__ void mfma16_first(v4f& acc, const v8i& first, const v
     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:%3 blgp:%4" : "=a"(acc) : "v"(first), "v"(second), "n"(F1), "n"(F2));
 }
 
-// Scales the 8 x 8 tiles of 16 x 16 accumulators, adds the bias, converts and writes C.
+// One accumulator register into a vector register, as an instruction of its own: it stays where it is written
+// relative to the MFMAs (also volatile asm).  Left to the compiler, which takes the MFMAs for ordinary
+// instructions, the copy may be placed right behind the MFMA that produces the value, where it reads the old one.
+__device__ __forceinline__ float acc_read(float a) {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+
+// The epilogue: scales the 8 x 8 tiles of 16 x 16 accumulators, adds the bias, converts and writes C.
 // acc[tj][ti] as left by MFMA(first = Bt rows, second = A rows): lane holds row ti*16 + lane%16
 // and the four columns tj*16 + 4*(lane/16) + e of its wave's 128 x 128 quarter.
+//
+// 16-bit outputs go straight from the registers, one `piece` = one store instruction at a time, so that the
+// kernel can slot the pieces of a finished row of tiles between the MFMAs of the next row in its last step.
+// A lane holds 4 neighbouring columns of a row (8 bytes) of each accumulator tile; v_permlane16_swap between the
+// tiles tj = 2p and 2p + 1 trades the odd 16-lane rows of the first for the even ones of the second, after which
+// every lane holds 8 neighbouring columns (lq even: columns 4 lq .. 4 lq + 7 of tile 2p; lq odd: columns
+// 4 (lq - 1) .. + 7 of tile 2p + 1) and one 16-byte store per lane writes 64 contiguous bytes of 16 rows.
+// (Staging the tile through LDS for 256-byte row segments takes the same time and needs the slabs to be free.)
 template <int C_DT>
-__device__ __forceinline__ void store_c_tile16(v4f (&acc)[8][8], int m0, int n0, int M, int N, float inv,
-                                               void* __restrict__ C, int64_t ldc, const void* __restrict__ bias,
-                                               int c_vec_ok) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int lm = lane & 15, lq = lane >> 4;
-    const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
+struct Epilogue16 {
+    int M, N, c_vec_ok, lq, row0, col0, wcol0;
+    float inv;
+    int64_t ldc;
+    void* C;
+    const void* bias;
+    float bv[8][4];
 
-    if constexpr (C_DT == F8MI_FP32) {
-        float* Cf = (float*)C;
-#pragma unroll
-        for (int tj = 0; tj < 8; tj++) {
-            const int col = wcol0 + tj * 16 + 4 * lq;
-            float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (bias) {
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (col + r < N) bv[r] = load_bias<C_DT>(bias, col + r);
-            }
-#pragma unroll
-            for (int ti = 0; ti < 8; ti++) {
-                const int row = wrow0 + ti * 16 + lm;
-                if (row >= M || col >= N) continue;
-                float v[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++) v[r] = acc[tj][ti][r] * inv + bv[r];
-                float* dst = Cf + (int64_t)row * ldc + col;
-                if (c_vec_ok && col + 4 <= N) {
-                    *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        if (col + r < N) dst[r] = v[r];
-                }
-            }
-        }
-    } else {
-        // 16-bit outputs straight from the registers.  A lane holds 4 neighbouring columns of a row (8 bytes) of
-        // each accumulator tile; v_permlane16_swap between the tiles tj = 2p and 2p + 1 trades the odd 16-lane rows
-        // of the first for the even ones of the second, after which every lane holds 8 neighbouring columns
-        // (lq even: columns 4 lq .. 4 lq + 7 of tile 2p; lq odd: columns 4 (lq - 1) .. + 7 of tile 2p + 1) and one
-        // 16-byte store per lane writes 64 contiguous bytes of 16 rows.  (Staging the tile through LDS for 256-byte
-        // row segments took twice the time: with one wave per SIMD nothing hides the round trip.)
-        uint16_t* Ch = (uint16_t*)C;
-        float bv[8][4];
+    __device__ __forceinline__ Epilogue16(int m0, int n0, int M_, int N_, float inv_, void* C_, int64_t ldc_, const void* bias_,
+                                          int c_vec_ok_)
+        : M(M_), N(N_), c_vec_ok(c_vec_ok_), inv(inv_), ldc(ldc_), C(C_), bias(bias_) {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        lq = lane >> 4;
+        wcol0 = n0 + (wave & 1) * 128;
+        row0 = m0 + (wave >> 1) * 128 + (lane & 15);
+        col0 = wcol0 + (lq & 1) * 16 + (lq >> 1) * 8;  // of the lane's 8 columns in the first pair of tiles
+    }
+
+    __device__ __forceinline__ void load_bias_row() {
 #pragma unroll
         for (int tj = 0; tj < 8; tj++) {
 #pragma unroll
@@ -92,31 +83,70 @@ __device__ __forceinline__ void store_c_tile16(v4f (&acc)[8][8], int m0, int n0,
                 bv[tj][r] = (bias && col < N) ? load_bias<C_DT>(bias, col) : 0.f;
             }
         }
-        const int col_l = (lq & 1) * 16 + (lq >> 1) * 8;  // inside the 32 columns of a pair of tiles
+    }
+
+    // rows ti*16 .. +15, columns tp*32 .. +31 of the wave's quarter (C_DT: bf16 or fp16); every lane must call it
+    __device__ __forceinline__ void piece(v4f (&acc)[8][8], int ti, int tp) {
+        const int te = 2 * tp, to = 2 * tp + 1;
+        float e[4], o[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) e[r] = acc_read(acc[te][ti][r]);
+#pragma unroll
+        for (int r = 0; r < 4; r++) o[r] = acc_read(acc[to][ti][r]);
+        const uint32_t x0 = pack2<C_DT>(e[0] * inv + bv[te][0], e[1] * inv + bv[te][1]);
+        const uint32_t x1 = pack2<C_DT>(e[2] * inv + bv[te][2], e[3] * inv + bv[te][3]);
+        const uint32_t y0 = pack2<C_DT>(o[0] * inv + bv[to][0], o[1] * inv + bv[to][1]);
+        const uint32_t y1 = pack2<C_DT>(o[2] * inv + bv[to][2], o[3] * inv + bv[to][3]);
+        const auto s0 = __builtin_amdgcn_permlane16_swap(x0, y0, false, false);
+        const auto s1 = __builtin_amdgcn_permlane16_swap(x1, y1, false, false);
+        const int row = row0 + ti * 16, col = col0 + tp * 32;
+        if (row < M && col < N) {
+            uint16_t* dst = (uint16_t*)C + (int64_t)row * ldc + col;
+            if (c_vec_ok && col + 8 <= N) {
+                *(uint4*)dst = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+            } else {
+                const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    if (col + i < N) dst[i] = (uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+            }
+        }
+    }
+};
+
+// fp32 outputs: a lane's 4 columns are 16 bytes already
+__device__ __forceinline__ void store_c_tile16_fp32(v4f (&acc)[8][8], int m0, int n0, int M, int N, float inv,
+                                                    void* __restrict__ C, int64_t ldc, const void* __restrict__ bias,
+                                                    int c_vec_ok) {
+    constexpr int C_DT = F8MI_FP32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lm = lane & 15, lq = lane >> 4;
+    const int wrow0 = m0 + wm * 128, wcol0 = n0 + wn * 128;
+    float* Cf = (float*)C;
+#pragma unroll
+    for (int tj = 0; tj < 8; tj++) {
+        const int col = wcol0 + tj * 16 + 4 * lq;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias) {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (col + r < N) bv[r] = load_bias<C_DT>(bias, col + r);
+        }
 #pragma unroll
         for (int ti = 0; ti < 8; ti++) {
             const int row = wrow0 + ti * 16 + lm;
+            if (row >= M || col >= N) continue;
+            float v[4];
 #pragma unroll
-            for (int tp = 0; tp < 4; tp++) {
-                const int te = 2 * tp, to = 2 * tp + 1;
-                const uint32_t x0 = pack2<C_DT>(acc[te][ti][0] * inv + bv[te][0], acc[te][ti][1] * inv + bv[te][1]);
-                const uint32_t x1 = pack2<C_DT>(acc[te][ti][2] * inv + bv[te][2], acc[te][ti][3] * inv + bv[te][3]);
-                const uint32_t y0 = pack2<C_DT>(acc[to][ti][0] * inv + bv[to][0], acc[to][ti][1] * inv + bv[to][1]);
-                const uint32_t y1 = pack2<C_DT>(acc[to][ti][2] * inv + bv[to][2], acc[to][ti][3] * inv + bv[to][3]);
-                const auto s0 = __builtin_amdgcn_permlane16_swap(x0, y0, false, false);  // all lanes take part
-                const auto s1 = __builtin_amdgcn_permlane16_swap(x1, y1, false, false);
-                const int col = wcol0 + tp * 32 + col_l;
-                if (row < M && col < N) {
-                    uint16_t* dst = Ch + (int64_t)row * ldc + col;
-                    if (c_vec_ok && col + 8 <= N) {
-                        *(uint4*)dst = make_uint4(s0[0], s1[0], s0[1], s1[1]);
-                    } else {
-                        const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
+            for (int r = 0; r < 4; r++) v[r] = acc_read(acc[tj][ti][r]) * inv + bv[r];
+            float* dst = Cf + (int64_t)row * ldc + col;
+            if (c_vec_ok && col + 4 <= N) {
+                *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
 #pragma unroll
-                        for (int i = 0; i < 8; i++)
-                            if (col + i < N) dst[i] = (uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
-                    }
-                }
+                for (int r = 0; r < 4; r++)
+                    if (col + r < N) dst[r] = v[r];
             }
         }
     }
@@ -321,6 +351,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
     // step's start with step t+2); 1: last but one (nothing left to fetch); 2: last step; 3: step 0 (as 0,
     // and the accumulators start from zero).
     int a_slab = 0;  // slab of A of this step; step t+2 goes to the slab before it in the rotation
+    constexpr bool EPI16 = C_DT != F8MI_FP32;
+    Epilogue16<EPI16 ? C_DT : F8MI_BF16> epi(m0, n0, M, N, inv, C, ldc, bias, c_vec_ok);
     auto step = [&](auto parity, auto mode) __attribute__((always_inline)) {
         constexpr int P = decltype(parity)::value;
         constexpr bool FIRST = decltype(mode)::value == 3;
@@ -336,6 +368,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
         }
         // Everything that is not an MFMA sits in a fixed slot between two MFMAs (each keeps the matrix
         // core busy for 32 cycles): one fragment (two 16-byte LDS reads) or one DMA at a time.
+        // The last step has neither; there the finished row of accumulator tiles (ti - 1: its last MFMA was issued
+        // eight MFMAs before the first read) is scaled, converted and stored under the MFMAs of row ti.
+        if (MODE == 2 && EPI16) epi.load_bias_row();
 #pragma unroll
         for (int ti = 0; ti < 8; ti++) {
             if (ti == 6 && MODE < 2) {
@@ -352,6 +387,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
                 if (FIRST) mfma16_first<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
                 else mfma16<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
                 F8MI_SCHED_FENCE();
+                if (MODE == 2 && EPI16 && ti >= 1 && (tj & 1) == 1) {
+                    epi.piece(acc, ti - 1, tj >> 1);
+                    F8MI_SCHED_FENCE();
+                }
                 if (MODE == 0 && (tj & 3) == 0) {
                     // 16 DMAs over the 64 MFMAs, one after every fourth: A slab first, then Bt.  (Packed into
                     // the first half of the step they cost 3 % more time: the four waves share one load unit.)
@@ -389,10 +428,15 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
         step(c0, c1);
         step(c1, c2);
     }
-    // the last MFMAs are still in the pipeline (8 passes): keep the accumulator reads away from them
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-
-    store_c_tile16<C_DT>(acc, m0, n0, M, N, inv, C, ldc, bias, c_vec_ok);
+    // the last MFMAs are still in the pipeline (8 passes): keep the accumulator reads away from them.  (No DMA is
+    // outstanding: the last but one step waited for all of them.)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    if constexpr (EPI16) {
+#pragma unroll
+        for (int tp = 0; tp < 4; tp++) epi.piece(acc, 7, tp);
+    } else {
+        store_c_tile16_fp32(acc, m0, n0, M, N, inv, C, ldc, bias, c_vec_ok);
+    }
 }
 
 template <int AF, int BF, int C_DT, bool ODD, bool A_TR, bool B_TR>
