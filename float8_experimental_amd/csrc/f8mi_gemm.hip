@@ -288,6 +288,24 @@ static int gemm_impl() {
     return v;
 }
 
+// An output whose last round of 256 x 256 tiles would leave most CUs idle (at most 128 tiles in it) is split by
+// rows: the tile rows that fill whole rounds go to the large-tile kernel, the rest to a 128-row-tile kernel that
+// spreads them over all CUs (same accumulation order, so no output bit depends on the split).  Returns the number
+// of tile rows for the large tiles (0: no split) and which 128-row tile takes the rest.
+struct RowSplit { int64_t rows_large; int mid; };
+static RowSplit split_last_round(int64_t tiles_m, int64_t tiles_n, int64_t k) {
+    const int64_t tiles = tiles_m * tiles_n, per_round = 256;
+    if (tiles <= per_round || tiles % per_round == 0) return {0, 0};
+    const int64_t rows_large = (tiles / per_round) * per_round / tiles_n;
+    if (rows_large < 1 || rows_large >= tiles_m) return {0, 0};
+    const int mid = use_mid_tiles((tiles_m - rows_large) * tiles_n, k);
+    if (!mid) return {0, 0};
+    // in rounds of the large-tile kernel: a round of 128 x 128 tiles takes about 0.5, one of 128 x 256 tiles 0.8 (measured)
+    const double cost = (double)((rows_large * tiles_n + per_round - 1) / per_round) + (mid == 1 ? 0.5 : 0.8);
+    if (cost > (double)((tiles + per_round - 1) / per_round) - 0.1) return {0, 0};
+    return {rows_large, mid};
+}
+
 extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fmt, int64_t ldb, int64_t m,
                             int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c,
                             int c_dtype, int64_t ldc, const void* bias_dev, void* stream_) {
@@ -312,7 +330,8 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     // Which kernel (the k-blocked entry point below decides the same way, so both give the same bits):
     //   aligned, K % 128 == 0:  up to 256 rows            -> few-row kernel (Bt streamed once, k split over waves)
     //                           up to 64 / 128 large tiles -> 128 x 128 / 128 x 256 tiles
-    //                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA
+    //                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA (the tile rows of a
+    //                                                        sparse last round: 128-row tiles, see split_last_round)
     //   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
     //   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
     if (aligned && M <= SKINNY_MAX_M && K % 128 == 0 && K > 0 && gemm_impl() == 0)
@@ -321,8 +340,17 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
         return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
     // F8MI_GEMM_IMPL=staged forces the register-staged kernel, =dma32 the 32x32x64 LDS-DMA kernel (comparison runs)
     if (aligned && K >= 384 && K % 64 == 0 && gemm_impl() != 1) {
-        if (K % 128 == 0 && gemm_impl() != 2)
+        if (K % 128 == 0 && gemm_impl() != 2) {
+            if (const RowSplit sp = gemm_impl() == 0 ? split_last_round(tiles_m, tiles_n, K) : RowSplit{0, 0}; sp.rows_large) {
+                const int m1 = (int)(sp.rows_large * BM);
+                if (int rc = launch_gemm_dma16(a_fmt, b_fmt, c_dtype, dim3((unsigned)(sp.rows_large * tiles_n)), stream, A, lda, 64, B, ldb, 64, m1, N, K,
+                                               scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)sp.rows_large, (int)tiles_n, c_vec_ok))
+                    return rc;
+                return launch_gemm_mid(a_fmt, b_fmt, c_dtype, sp.mid == 2, stream, A + (int64_t)m1 * lda, lda, 64, B, ldb, 64, M - m1, N, K, scale_a_dev,
+                                       scale_b_dev, (uint8_t*)c + (int64_t)m1 * ldc * csz, ldc, bias_dev, c_vec_ok);
+            }
             return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+        }
         return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     }
     if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_gemm1<0, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
@@ -354,9 +382,20 @@ extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_f
     if (const int mid = gemm_impl() == 0 ? use_mid_tiles(tiles_m * tiles_n, k) : 0)
         return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n, (int)k,
                                scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
-    if (k % 128 == 0 && gemm_impl() != 2)
+    if (k % 128 == 0 && gemm_impl() != 2) {
+        if (const RowSplit sp = gemm_impl() == 0 ? split_last_round(tiles_m, tiles_n, k) : RowSplit{0, 0}; sp.rows_large) {
+            // rows m1 .. m of a k-blocked operand start m1 * 64 bytes in; the distance between 64-deep blocks stays m * 64
+            const int64_t m1 = sp.rows_large * BM;
+            if (int rc = launch_gemm_dma16(a_fmt, b_fmt, c_dtype, dim3((unsigned)(sp.rows_large * tiles_n)), stream, (const uint8_t*)a, 64, m * 64,
+                                           (const uint8_t*)bt, 64, n * 64, (int)m1, (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev,
+                                           (int)sp.rows_large, (int)tiles_n, c_vec_ok))
+                return rc;
+            return launch_gemm_mid(a_fmt, b_fmt, c_dtype, sp.mid == 2, stream, (const uint8_t*)a + m1 * 64, 64, m * 64, (const uint8_t*)bt, 64, n * 64,
+                                   (int)(m - m1), (int)n, (int)k, scale_a_dev, scale_b_dev, (uint8_t*)c + m1 * ldc * csz, ldc, bias_dev, c_vec_ok);
+        }
         return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
                                  (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    }
     return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
                            (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
 }

@@ -439,6 +439,27 @@ def test_gemm_mid_tile_kernel_shapes(nat, m, n, k, out_dt):
     _gemm_check(nat, m, n, k, fm[0], fm[1], out_dt, seed=m + n + k, bias=(n % 2 == 0))
 
 
+# More than one round of 256 x 256 tiles with few tiles in the last one: the last tile rows go to a 128-row-tile kernel.
+@pytest.mark.parametrize("m,n,k,m_pad", [(4352, 4096, 512, 8192),      # 272 tiles: 16 of them as 128 x 128 tiles
+                                         (8500, 2048, 384, 16384),     # ragged last tile row
+                                         (6144, 4096, 640, 8192),      # 384 tiles: 128 of them as 128 x 256 tiles
+                                         (16640, 4000, 384, 20480)])   # four full rounds, then 16 tiles; ragged columns
+def test_gemm_split_of_a_sparse_last_round_changes_no_bit(nat, m, n, k, m_pad):
+    """Reference: the same rows inside a matrix padded with zero rows to whole rounds, which the large-tile kernel
+    computes alone."""
+    a = _rand_fp8((m, k), torch.float8_e4m3fn, m + k, 4.0).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e5m2, n + k, 4.0).to(DEV)
+    sa, sb = torch.tensor(0.5, device=DEV), torch.tensor(4.0, device=DEV)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 3).to(torch.bfloat16).to(DEV)
+    assert (m_pad // 256) * ((n + 255) // 256) % 256 == 0
+    a_pad = torch.cat([a.view(torch.uint8), torch.zeros(m_pad - m, k, dtype=torch.uint8, device=DEV)]).view(a.dtype)
+    for out_dt, b in ((torch.bfloat16, bias), (torch.float32, None)):
+        want = nat.gemm_nt(a_pad, sa, bt, sb, out_dt, bias=b)[:m]
+        assert torch.equal(nat.gemm_nt(a, sa, bt, sb, out_dt, bias=b), want)
+        assert torch.equal(nat.gemm_nt_kb(_to_kb(a), sa, _to_kb(bt), sb, out_dt, bias=b), want)
+    _gemm_check(nat, m, n, k, "e4m3", "e5m2", torch.bfloat16, seed=m + n, bias=True)
+
+
 @pytest.mark.parametrize("m,n,k", [(300, 520, 1024), (1000, 264, 2048), (512, 1024, 384), (1100, 4500, 640)])
 def test_gemm_mid_tile_kernel_equals_the_large_tile_kernel_bitwise(nat, m, n, k):
     """The same rows of A inside a matrix tall enough for the 256 x 256-tile kernel: identical bits (same accumulation
