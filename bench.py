@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this script, each scaled by the same counter's reading for a
 # 1 GiB device copy (x2.0 and x1.0); the summary is profiles/bench_llama70b_gemm_hbm_traffic_pmc.txt.
 # Only meaningful at the default --m.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 5.69e9
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 5.74e9
 
 
 def parse():
