@@ -216,3 +216,37 @@ def test_inductor_backend_if_it_is_usable_here(f8):
     # the other side of an fp8 rounding boundary: agreement is statistical, far above the float8 noise floor
     for a, b in zip(got, want):
         assert f8.float8_utils.compute_error(b.float(), a.float()).item() > 25
+
+
+def test_inductor_backend_with_delayed_scaling(f8):
+    """The amax buffers are graph inputs that the compiled code mutates; the sync stays an eager call between steps."""
+    torch.manual_seed(7)
+    D = f8.CastConfig(f8.ScalingType.DELAYED)
+    cfg = f8.Float8LinearConfig(cast_config_input=D, cast_config_weight=D, cast_config_grad_output=D,
+                                enable_amax_init=False, enable_pre_and_post_forward=False)
+    base = nn.Sequential(nn.Linear(512, 448, bias=True), nn.SiLU(), nn.Linear(448, 384, bias=False)).to(DEV, dtype=torch.bfloat16)
+    a, b = copy.deepcopy(base), copy.deepcopy(base)
+    f8.convert_to_float8_training(a, config=cfg)
+    f8.convert_to_float8_training(b, config=cfg)
+    torch._dynamo.reset()
+    cb = torch.compile(b, backend="inductor", fullgraph=True)
+    for it in range(3):
+        x = torch.randn(64, 512, device=DEV, dtype=torch.bfloat16) * 1.5 ** it
+        dy = torch.randn(64, 384, device=DEV, dtype=torch.bfloat16)
+        f8.sync_float8_amax_and_scale_history(a)
+        f8.sync_float8_amax_and_scale_history(b)
+        want = _run(a, x, dy)
+        try:
+            got = _run(cb, x, dy)
+        except Exception as e:
+            if it == 0:
+                pytest.skip(f"inductor cannot generate code here: {type(e).__name__}")
+            raise
+        # the first layer sees identical inputs: its recorded amaxes agree exactly; behind the compiler's own SiLU the
+        # values differ in the last bf16 bit (see the dynamic-scaling inductor test), so the rest agrees statistically
+        assert torch.equal(a[0].fp8_amax_input, b[0].fp8_amax_input) and torch.equal(a[0].fp8_amax_weight, b[0].fp8_amax_weight)
+        for (name, b1), (_, b2) in zip(a.named_buffers(), b.named_buffers()):
+            torch.testing.assert_close(b1, b2, rtol=0.02, atol=0)
+        if it > 0:  # iteration 0 runs on the default scale 1.0: small values underflow in fp8 and there is little signal
+            for u, v in zip(got, want):
+                assert f8.float8_utils.compute_error(v.float(), u.float()).item() > 20
