@@ -328,13 +328,14 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     const uint8_t* B = (const uint8_t*)bt;
     const int M = (int)m, N = (int)n, K = (int)k;
     // Which kernel (the k-blocked entry point below decides the same way, so both give the same bits):
-    //   aligned, K % 128 == 0:  up to 256 rows            -> few-row kernel (Bt streamed once, k split over waves)
+    //   aligned, K % 128 == 0:  up to 128 rows, or up to 256 and a narrow Bt (use_skinny)
+    //                                                     -> few-row kernel (Bt streamed once per 128 rows, k split over waves)
     //                           up to 64 / 128 large tiles -> 128 x 128 / 128 x 256 tiles
     //                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA (the tile rows of a
     //                                                        sparse last round: 128-row tiles, see split_last_round)
     //   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
     //   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
-    if (aligned && M <= SKINNY_MAX_M && K % 128 == 0 && K > 0 && gemm_impl() == 0)
+    if (aligned && use_skinny(M, N, K) && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
     if (const int mid = (aligned && gemm_impl() == 0) ? use_mid_tiles(tiles_m * tiles_n, K) : 0)
         return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
@@ -376,7 +377,7 @@ extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_f
     const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
-    if (m <= SKINNY_MAX_M && k % 128 == 0 && gemm_impl() == 0)
+    if (use_skinny(m, n, k) && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n,
                                   (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
     if (const int mid = gemm_impl() == 0 ? use_mid_tiles(tiles_m * tiles_n, k) : 0)

@@ -185,6 +185,18 @@ inline int use_mid_tiles(int64_t tiles_256, int64_t k) {
 // few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands.  One limit for row-major and
 // k-blocked operands, so that the two entry points keep giving the same bits.
 constexpr int SKINNY_MAX_M = 256;
+// From 129 rows on the few-row kernel passes over Bt twice, and a wide Bt is then cheaper as one round (or two) of
+// 128-row tiles.  Estimates per unit of k, in ns, fitted to measurements at 144 - 256 rows (n x k: 4096 x 4096 14 against
+// 20 us for the tiles, 4096 x 14336 36 / 60, 8192 x 8192 41 - 48 / 37, 14336 x 4096 39 - 47 / 22, 28672 x 8192 119 - 143 / 59).
+// Depends on the shape only, so the row-major and the k-blocked entry point agree.
+inline bool use_skinny(int64_t m, int64_t n, int64_t k) {
+    if (m > SKINNY_MAX_M || k <= 0 || k % 128 != 0) return false;
+    if (m <= 128) return true;
+    const double tiles = 2.0 * (double)((n + 127) / 128);
+    const double t_tiles = 4.4 * (0.0035 * tiles > 1.0 ? 0.0035 * tiles : 1.0);
+    const double t_skinny = 4000.0 / (double)k + 0.0006 * (double)n;
+    return t_skinny <= t_tiles;
+}
 int launch_gemm_skinny(int a_fmt, int b_fmt, int c_dtype, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                        const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                        int64_t ldc, const void* bias);
