@@ -460,7 +460,8 @@ def test_gemm_split_of_a_sparse_last_round_changes_no_bit(nat, m, n, k, m_pad):
     _gemm_check(nat, m, n, k, "e4m3", "e5m2", torch.bfloat16, seed=m + n, bias=True)
 
 
-@pytest.mark.parametrize("m,n,k", [(300, 520, 1024), (1000, 264, 2048), (512, 1024, 384), (1100, 4500, 640)])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 1024), (1000, 264, 2048), (512, 1024, 384), (1100, 4500, 640),
+                                   (200, 8192, 512)])  # 129 - 256 rows and a wide Bt: the 128-row tiles, not the few-row kernel
 def test_gemm_mid_tile_kernel_equals_the_large_tile_kernel_bitwise(nat, m, n, k):
     """The same rows of A inside a matrix tall enough for the 256 x 256-tile kernel: identical bits (same accumulation
     order), row-major and k-blocked."""
