@@ -161,22 +161,14 @@ def linear_dynamic(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return linear(x, weight)
 
 
-_sync_tables = {}
-
-
 @torch.library.custom_op("f8mi::sync", mutates_args=("scales",))
 def sync(amaxes: List[torch.Tensor], histories: List[torch.Tensor], scales: List[torch.Tensor], is_e5m2: List[bool],
          orig_is_fp16: bool) -> None:
     """The delayed-scaling sync of all listed buffers as one node (and one kernel launch): for each i,
     ``scales[i] = fmax / max(amaxes[i], histories[i][:-1])`` in the reference's rounding
     (float8_linear_utils.py:287-319).  No autograd: the buffers carry none."""
-    key = tuple(t.data_ptr() for group in (amaxes, histories, scales) for t in group)
-    table = _sync_tables.get(key)
-    if table is None:
-        if len(_sync_tables) > 64:
-            _sync_tables.clear()
-        rows = [(a, h, s, e5m2_dtype if e else e4m3_dtype) for a, h, s, e in zip(amaxes, histories, scales, is_e5m2)]
-        table = _sync_tables[key] = _native.sync_table(rows, amaxes[0].device)
+    table = _native.sync_table_cached((a, h, s, e5m2_dtype if e else e4m3_dtype)
+                                      for a, h, s, e in zip(amaxes, histories, scales, is_e5m2))
     _native.sync(table, histories[0].numel(), orig_is_fp16, writeback_history=False)
 
 

@@ -447,6 +447,22 @@ def sync_table(entries, device: torch.device) -> torch.Tensor:
     return torch.tensor(rows, dtype=torch.int64, device="cpu").to(device)
 
 
+_sync_tables = {}
+
+
+def sync_table_cached(entries) -> torch.Tensor:
+    """``sync_table`` of the same buffers as last time without rebuilding it: the table is rebuilt only when a
+    buffer has moved (``.to()``, ``load_state_dict`` into new storage, ...)."""
+    entries = list(entries)
+    key = tuple((a.data_ptr(), h.data_ptr(), s.data_ptr(), _F8[f8]) for a, h, s, f8 in entries)
+    hit = _sync_tables.get(key)
+    if hit is None:
+        if len(_sync_tables) > 64:
+            _sync_tables.clear()
+        hit = _sync_tables[key] = sync_table(entries, entries[0][0].device)
+    return hit
+
+
 def sync(table: torch.Tensor, hist_len: int, orig_is_fp16: bool, writeback_history: bool = False) -> None:
     _require_gpu(table, "table")
     assert table.dtype == torch.int64 and table.dim() == 2 and table.shape[1] == 4 and table.is_contiguous()

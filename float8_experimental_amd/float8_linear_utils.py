@@ -70,25 +70,12 @@ def get_float8_layers(model: torch.nn.Module) -> List[Float8Linear]:
     return [m for m in model.modules() if isinstance(m, Float8Linear)]
 
 
-_sync_tables = {}
-
-
 def _sync_table(fp8_layers) -> torch.Tensor:
-    """Device table of (amax, history, scale, format) pointers for all 3L buffers, rebuilt only when a
-    buffer has moved (``.to()``, ``load_state_dict`` into new storage, ...)."""
-    bufs = []
-    for child in fp8_layers:
-        for kind, f8 in _KINDS:
-            bufs.append((getattr(child, f"fp8_amax_{kind}"), getattr(child, f"fp8_amax_history_{kind}"),
-                         getattr(child, f"fp8_scale_{kind}"), f8))
-    key = tuple(t.data_ptr() for row in bufs for t in row[:3])
-    hit = _sync_tables.get(key)
-    if hit is None:
-        if len(_sync_tables) > 64:
-            _sync_tables.clear()
-        hit = _native.sync_table(bufs, bufs[0][0].device)
-        _sync_tables[key] = hit
-    return hit
+    """Device table of (amax, history, scale, format) pointers for all 3L buffers (cached while the buffers stay
+    where they are)."""
+    return _native.sync_table_cached(
+        (getattr(child, f"fp8_amax_{kind}"), getattr(child, f"fp8_amax_history_{kind}"), getattr(child, f"fp8_scale_{kind}"), f8)
+        for child in fp8_layers for kind, f8 in _KINDS)
 
 
 @torch.no_grad()
