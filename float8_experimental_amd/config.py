@@ -62,7 +62,8 @@ class Float8LinearConfig:
     enable_amax_init: bool = True
     # run the synced/initialised bookkeeping around forward
     enable_pre_and_post_forward: bool = True
-    # FSDP2 float8 all-gather of the weight: needs more than one GPU, not available in this build
+    # FSDP2 float8 all-gather of the weight: on one GPU nothing is gathered; the flag marks the weights whose
+    # scales precompute_float8_dynamic_scale_for_fsdp computes ahead of the forward pass
     enable_fsdp_float8_all_gather: bool = False
     # zero-pad the reduction dimension to a multiple of 16 before the GEMM; the kernel
     # here handles ragged shapes itself, so the flag is accepted and has no effect on results

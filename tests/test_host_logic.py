@@ -35,9 +35,10 @@ def cfg(i=DYN, w=DYN, g=DYN, **kw):
 
 
 def test_public_names_match_the_reference():
-    assert f8.__all__ == ["DelayedScalingConfig", "ScalingType", "Float8GemmConfig", "Float8LinearConfig", "CastConfig",
-                          "convert_to_float8_training", "linear_requires_sync", "sync_float8_amax_and_scale_history",
-                          "precompute_float8_dynamic_scale_for_fsdp"]
+    assert sorted(f8.__all__) == sorted([
+        "DelayedScalingConfig", "ScalingType", "Float8GemmConfig", "Float8LinearConfig", "CastConfig",
+        "convert_to_float8_training", "linear_requires_sync", "sync_float8_amax_and_scale_history",
+        "precompute_float8_dynamic_scale_for_fsdp"])
     for name in f8.__all__ + ["Float8Tensor", "Float8Linear", "GemmInputRole", "LinearMMConfig", "ScaledMMConfig"]:
         assert hasattr(f8, name)
 
