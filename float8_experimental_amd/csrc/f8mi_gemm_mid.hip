@@ -54,6 +54,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
     lid = xcd_contiguous_id(lid, gridDim.x);
     const int tm = lid % tiles_m, tn = lid / tiles_m;
     const int m0 = tm * MID_TILE_M, n0 = tn * Cfg::TILE_N;
+    // 1 / (sa * sb) for the epilogue, fetched before the main loop and kept in a scalar register
+    const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
+        int, __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev))));
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave >> 1, wn = wave & 1;
@@ -157,25 +160,25 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
 
     // ---- epilogue: MFMA(first = Bt rows, second = A rows) leaves lane l with row ti*16 + l%16 and the four
     // columns tj*16 + 4*(l/16) + e of the wave's 64 x (16 TJ)
-    const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
     const int lm = lane & 15, lq = lane >> 4;
+    const int wcol0 = n0 + wn * (TJ * 16);
+    if constexpr (C_DT == F8MI_FP32) {
 #pragma unroll
-    for (int tj = 0; tj < TJ; tj++) {
-        const int col = n0 + wn * (TJ * 16) + tj * 16 + 4 * lq;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bias) {
+        for (int tj = 0; tj < TJ; tj++) {
+            const int col = wcol0 + tj * 16 + 4 * lq;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (col + e < N) bv[e] = load_bias<C_DT>(bias, col + e);
-        }
+                for (int e = 0; e < 4; e++)
+                    if (col + e < N) bv[e] = load_bias<C_DT>(bias, col + e);
+            }
 #pragma unroll
-        for (int ti = 0; ti < 4; ti++) {
-            const int row = m0 + wm * 64 + ti * 16 + lm;
-            if (row >= M || col >= N) continue;
-            float v[4];
+            for (int ti = 0; ti < 4; ti++) {
+                const int row = m0 + wm * 64 + ti * 16 + lm;
+                if (row >= M || col >= N) continue;
+                float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = acc[tj][ti][e] * inv + bv[e];
-            if constexpr (C_DT == F8MI_FP32) {
+                for (int e = 0; e < 4; e++) v[e] = acc[tj][ti][e] * inv + bv[e];
                 float* dst = (float*)C + (int64_t)row * ldc + col;
                 if (c_vec_ok && col + 4 <= N) {
                     *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
@@ -184,16 +187,46 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
                     for (int e = 0; e < 4; e++)
                         if (col + e < N) dst[e] = v[e];
                 }
-            } else {
-                uint16_t* dst = (uint16_t*)C + (int64_t)row * ldc + col;
-                const uint32_t p0 = pack2<C_DT>(v[0], v[1]), p1 = pack2<C_DT>(v[2], v[3]);
-                if (c_vec_ok && col + 4 <= N) {
-                    *(uint2*)dst = make_uint2(p0, p1);
-                } else {
-                    const uint32_t w[2] = {p0, p1};
+            }
+        }
+    } else {
+        // 2-byte outputs: v_permlane16_swap between the accumulator tiles 2p and 2p + 1 trades the odd 16-lane rows of
+        // the first for the even ones of the second, which turns a lane's 4 + 4 columns of two tiles into 8
+        // neighbouring columns of one (lq even: columns 4 lq .. + 7 of tile 2p, lq odd: 4 (lq - 1) .. + 7 of tile
+        // 2p + 1): one 16-byte store per lane, 64 contiguous bytes per row and instruction.
+        float bv[TJ][4];
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (col + e < N) dst[e] = (uint16_t)((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        for (int tj = 0; tj < TJ; tj++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int col = wcol0 + tj * 16 + 4 * lq + e;
+                bv[tj][e] = (bias && col < N) ? load_bias<C_DT>(bias, col) : 0.f;
+            }
+        }
+        const int col_l = (lq & 1) * 16 + (lq >> 1) * 8;
+#pragma unroll
+        for (int ti = 0; ti < 4; ti++) {
+            const int row = m0 + wm * 64 + ti * 16 + lm;
+#pragma unroll
+            for (int tp = 0; tp < TJ / 2; tp++) {
+                const int te = 2 * tp, to = 2 * tp + 1;
+                const uint32_t x0 = pack2<C_DT>(acc[te][ti][0] * inv + bv[te][0], acc[te][ti][1] * inv + bv[te][1]);
+                const uint32_t x1 = pack2<C_DT>(acc[te][ti][2] * inv + bv[te][2], acc[te][ti][3] * inv + bv[te][3]);
+                const uint32_t y0 = pack2<C_DT>(acc[to][ti][0] * inv + bv[to][0], acc[to][ti][1] * inv + bv[to][1]);
+                const uint32_t y1 = pack2<C_DT>(acc[to][ti][2] * inv + bv[to][2], acc[to][ti][3] * inv + bv[to][3]);
+                const auto s0 = __builtin_amdgcn_permlane16_swap(x0, y0, false, false);  // every lane takes part
+                const auto s1 = __builtin_amdgcn_permlane16_swap(x1, y1, false, false);
+                const int col = wcol0 + tp * 32 + col_l;
+                if (row < M && col < N) {
+                    uint16_t* dst = (uint16_t*)C + (int64_t)row * ldc + col;
+                    if (c_vec_ok && col + 8 <= N) {
+                        *(uint4*)dst = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                    } else {
+                        const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
+#pragma unroll
+                        for (int e = 0; e < 8; e++)
+                            if (col + e < N) dst[e] = (uint16_t)((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+                    }
                 }
             }
         }
