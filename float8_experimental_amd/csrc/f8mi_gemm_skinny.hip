@@ -41,6 +41,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(
     int64_t ldc, const void* __restrict__ bias) {
     constexpr int SK_DEPTH = sk_depth(MT);
     // blockIdx.y: which block of 16 * MT rows of A (and C) this workgroup multiplies
+    // 1 / (sa * sb) for the epilogue: fetched first, so that the round trip to memory is over long before it is needed
+    const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
     const int m_base = blockIdx.y * (16 * MT);
     const int M = min(M_all - m_base, 16 * MT);
     A += (int64_t)m_base * lda;
@@ -109,7 +111,6 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(
     }
     __syncthreads();
 
-    const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
     for (int item = threadIdx.x; item < MT * SK_NT * 64; item += SK_THREADS) {
         const int tile = item >> 6, l = item & 63;
         float4 sum = part[0][tile][l];
