@@ -257,8 +257,8 @@ def tn_ok(m: int, k: int, n: int) -> bool:
     transposed operands (smaller outputs are faster from transposed copies through the 128 x 128-tile kernel)."""
     if not all(d % 128 == 0 and d >= KB_MIN_K for d in (m, k, n)):
         return False
-    tiles = lambda rows, cols: -(-rows // 256) * -(-cols // 256)
-    return tiles(m, k) > 64 and tiles(n, k) > 64
+    tiles = lambda rows, cols: -(-rows // 128) * -(-cols // 128)  # of 128 x 128: at most one per CU -> that kernel
+    return tiles(m, k) > 256 and tiles(n, k) > 256
 
 
 def kblock_ok(k: int) -> bool:

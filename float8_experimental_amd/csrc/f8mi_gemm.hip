@@ -298,7 +298,7 @@ static RowSplit split_last_round(int64_t tiles_m, int64_t tiles_n, int64_t k) {
     if (tiles <= per_round || tiles % per_round == 0) return {0, 0};
     const int64_t rows_large = (tiles / per_round) * per_round / tiles_n;
     if (rows_large < 1 || rows_large >= tiles_m) return {0, 0};
-    const int mid = use_mid_tiles((tiles_m - rows_large) * tiles_n, k);
+    const int mid = use_mid_tiles((tiles_m - rows_large) * BM, tiles_n * BN, k);
     if (!mid) return {0, 0};
     // in rounds of the large-tile kernel: a round of 128 x 128 tiles takes about 0.5, one of 128 x 256 tiles 0.8 (measured)
     const double cost = (double)((rows_large * tiles_n + per_round - 1) / per_round) + (mid == 1 ? 0.5 : 0.8);
@@ -328,16 +328,16 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     const uint8_t* B = (const uint8_t*)bt;
     const int M = (int)m, N = (int)n, K = (int)k;
     // Which kernel (the k-blocked entry point below decides the same way, so both give the same bits):
-    //   aligned, K % 128 == 0:  up to 128 rows, or up to 256 and a narrow Bt (use_skinny)
+    //   aligned, K % 128 == 0:  up to 16 rows, or up to 256 and a narrow Bt (use_skinny)
     //                                                     -> few-row kernel (Bt streamed once per 128 rows, k split over waves)
-    //                           up to 64 / 128 large tiles -> 128 x 128 / 128 x 256 tiles
+    //                           up to 256 tiles of 128 x 128 / 128 x 256 -> those
     //                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA (the tile rows of a
     //                                                        sparse last round: 128-row tiles, see split_last_round)
     //   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
     //   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
     if (aligned && use_skinny(M, N, K) && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
-    if (const int mid = (aligned && gemm_impl() == 0) ? use_mid_tiles(tiles_m * tiles_n, K) : 0)
+    if (const int mid = (aligned && gemm_impl() == 0) ? use_mid_tiles(M, N, K) : 0)
         return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
     // F8MI_GEMM_IMPL=staged forces the register-staged kernel, =dma32 the 32x32x64 LDS-DMA kernel (comparison runs)
     if (aligned && K >= 384 && K % 64 == 0 && gemm_impl() != 1) {
@@ -380,7 +380,7 @@ extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_f
     if (use_skinny(m, n, k) && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n,
                                   (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
-    if (const int mid = gemm_impl() == 0 ? use_mid_tiles(tiles_m * tiles_n, k) : 0)
+    if (const int mid = gemm_impl() == 0 ? use_mid_tiles(m, n, k) : 0)
         return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n, (int)k,
                                scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
     if (k % 128 == 0 && gemm_impl() != 2) {

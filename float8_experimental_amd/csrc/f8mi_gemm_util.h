@@ -19,7 +19,6 @@ constexpr int EPI_BYTES = 4 * 128 * EPI_PITCH;
 constexpr int GEMM_LDS = 2 * STAGE_BYTES > EPI_BYTES ? 2 * STAGE_BYTES : EPI_BYTES;
 constexpr int GROUP_M = 8;
 constexpr int NUM_XCD = 8;
-constexpr int MID_MAX_TILES_256 = 64;
 
 // Consecutive workgroup ids go to the 8 XCDs round-robin.  Re-deals them so that XCD x (ids x, x+8, ...) works on
 // a contiguous run of the tile order -- whatever the grid size: the first `grid % 8` XCDs get one workgroup more.
@@ -175,26 +174,37 @@ static int allow_big_lds(K kern, int bytes, std::atomic<uint64_t>& done_mask) {
 int launch_gemm_mid(int a_fmt, int b_fmt, int c_dtype, bool wide, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                     const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                     int64_t ldc, const void* bias, int c_vec_ok);
-// They take over while their own tiles number at most one per CU: up to 64 tiles of 256 x 256 the 128 x 128 ones,
-// up to 128 the 128 x 256 ones (with more, the large tiles win again: measured).
+// They take over while their own tiles number at most one per CU (with more, the large tiles win again: measured):
+// 128 x 128 tiles while at most 256 of them cover the output, else 128 x 256 tiles while 256 of those do.
 // Returns 0: large tiles, 1: 128 x 128, 2: 128 x 256.
-inline int use_mid_tiles(int64_t tiles_256, int64_t k) {
-    if (k % 128 != 0 || k < 128 || tiles_256 > 2 * MID_MAX_TILES_256) return 0;
-    return tiles_256 <= MID_MAX_TILES_256 ? 1 : 2;
+inline int use_mid_tiles(int64_t m, int64_t n, int64_t k) {
+    if (k % 128 != 0 || k < 128) return 0;
+    const int64_t row_tiles = (m + 127) / 128;
+    if (row_tiles * ((n + 127) / 128) <= 256) return 1;
+    if (row_tiles * ((n + 255) / 256) <= 256) return 2;
+    return 0;
 }
-// few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands.  One limit for row-major and
-// k-blocked operands, so that the two entry points keep giving the same bits.
+// few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands.
 constexpr int SKINNY_MAX_M = 256;
-// From 129 rows on the few-row kernel passes over Bt twice, and a wide Bt is then cheaper as one round (or two) of
-// 128-row tiles.  Estimates per unit of k, in ns, fitted to measurements at 144 - 256 rows (n x k: 4096 x 4096 14 against
-// 20 us for the tiles, 4096 x 14336 36 / 60, 8192 x 8192 41 - 48 / 37, 14336 x 4096 39 - 47 / 22, 28672 x 8192 119 - 143 / 59).
-// Depends on the shape only, so the row-major and the k-blocked entry point agree.
+// Up to 16 rows the few-row kernel always runs: it streams Bt once at memory speed.  With more rows every one of its
+// 32-column workgroups re-reads A from L2, and from 129 rows on it passes over Bt twice, so a wide Bt is cheaper
+// as one round (or two) of 128-row tiles, which take the same time for 1 or 128 rows.  Estimates in us, fitted to
+// measurements (rows, n x k: few-row / tiles): 128, 8192 x 8192: 27 / 37; 128, 28672 x 8192: 83 / 37; 64, 28672 x 8192:
+// 53 / 37; 144 - 256, 4096 x 4096: 14 / 20; 4096 x 14336: 36 / 60; 8192 x 8192: 41 - 48 / 37; 14336 x 4096: 39 - 47 / 22;
+// 28672 x 8192: 119 - 143 / 59.  Depends on the shape only, so the row-major and the k-blocked entry point agree.
 inline bool use_skinny(int64_t m, int64_t n, int64_t k) {
     if (m > SKINNY_MAX_M || k <= 0 || k % 128 != 0) return false;
-    if (m <= 128) return true;
-    const double tiles = 2.0 * (double)((n + 127) / 128);
-    const double t_tiles = 4.4 * (0.0035 * tiles > 1.0 ? 0.0035 * tiles : 1.0);
-    const double t_skinny = 4000.0 / (double)k + 0.0006 * (double)n;
+    if (m <= 16) return true;
+    const double passes = (double)((m + 127) / 128);
+    const double row_tiles = m > 128 ? 8.0 : (double)((m + 15) / 16);  // 16-row tiles of A per pass
+    // Bt at 6.5 TB/s from memory plus A (n / 32 workgroups x 16 row_tiles x k bytes) at 20 TB/s from L2
+    const double t_skinny = passes * (2.0 + (double)n * (double)k * (0.154 + 0.025 * row_tiles) * 1e-6);
+    // one round of 128 x 128 tiles: 4.4 ns per unit of k; of 128 x 256 tiles: 7.8 ns; of 256 x 256 tiles: 10.6 ns
+    const int64_t rt = (m + 127) / 128;
+    double t_tiles;
+    if (rt * ((n + 127) / 128) <= 256) t_tiles = 4.4e-3 * (double)k;
+    else if (rt * ((n + 255) / 256) <= 256) t_tiles = 7.8e-3 * (double)k;
+    else t_tiles = 10.6e-3 * (double)k * (double)((((m + 255) / 256) * ((n + 255) / 256) + 255) / 256);
     return t_skinny <= t_tiles;
 }
 int launch_gemm_skinny(int a_fmt, int b_fmt, int c_dtype, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,

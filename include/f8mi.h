@@ -132,8 +132,8 @@ int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtyp
  * (float8_ops.py:158-190).  Both operands are contiguous along k (A row-major,
  * B column-major in the reference's words): forward x*W^T, grad_input dY*W and
  * grad_weight dY^T*x all have this form once the transposed copies exist.
- * Any m, n, k >= 0 is accepted (ragged edges are handled in the kernel).  Up to 128 rows of A (up to 256
- * when Bt is narrow enough that two passes over it beat a round of 128-row tiles) with k % 128 == 0 take a
+ * Any m, n, k >= 0 is accepted (ragged edges are handled in the kernel).  Up to 16 rows of A (up to 256
+ * while streaming Bt once per 128 rows beats a round of 128-row tiles: a narrow Bt) with k % 128 == 0 take a
  * kernel that reads Bt at memory speed (an inference decode step); it sums the products in another order
  * than the tile kernels, so its results agree with theirs within the accumulation tolerance, not bit for bit.
  * Which kernel runs depends on (m, n, k) and alignment only.

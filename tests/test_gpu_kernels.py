@@ -429,10 +429,11 @@ def test_gemm_few_rows_kblocked_equals_row_major_bitwise(nat, m, n, k):
     assert torch.equal(sub, want[: max(1, m // 3)])
 
 
-# Outputs of few 256 x 256 tiles (more than 256 rows, k % 128 == 0) take the 128 x 128-tile kernel (at most 64 of them) or
-# the 128 x 256-tile kernel (65 to 128; the last three cases).
+# Outputs that at most 256 tiles of 128 x 128 or of 128 x 256 cover (k % 128 == 0), unless the few-row kernel is
+# estimated to be faster, take those tiles.
 @pytest.mark.parametrize("m,n,k", [(257, 128, 128), (300, 520, 1024), (512, 1000, 256), (1024, 2048, 640), (384, 8192, 2048),
-                                   (4099, 500, 1152), (1024, 8192, 1024), (1000, 5000, 384), (2049, 3000, 128)])
+                                   (4099, 500, 1152), (1024, 8192, 1024), (1000, 5000, 384), (2049, 3000, 128),
+                                   (64, 28672, 512), (20, 16384, 256)])  # few rows, wide Bt: one partial row of tiles
 @pytest.mark.parametrize("out_dt", [torch.bfloat16, torch.float32])
 def test_gemm_mid_tile_kernel_shapes(nat, m, n, k, out_dt):
     fm = [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2"), ("e5m2", "e5m2")][(m + n + k // 128) % 4]
@@ -461,7 +462,8 @@ def test_gemm_split_of_a_sparse_last_round_changes_no_bit(nat, m, n, k, m_pad):
 
 
 @pytest.mark.parametrize("m,n,k", [(300, 520, 1024), (1000, 264, 2048), (512, 1024, 384), (1100, 4500, 640),
-                                   (200, 8192, 512)])  # 129 - 256 rows and a wide Bt: the 128-row tiles, not the few-row kernel
+                                   (200, 8192, 512),     # 129 - 256 rows and a wide Bt: the 128-row tiles, not the few-row kernel
+                                   (100, 16384, 384)])   # so do 17 - 128 rows when Bt is wide enough
 def test_gemm_mid_tile_kernel_equals_the_large_tile_kernel_bitwise(nat, m, n, k):
     """The same rows of A inside a matrix tall enough for the 256 x 256-tile kernel: identical bits (same accumulation
     order), row-major and k-blocked."""
