@@ -28,6 +28,8 @@ EXPORTS = (
     "f8mi_last_error",
     "f8mi_device_info",
     "f8mi_workspace_bytes",
+    "f8mi_gemm_nt_ws",
+    "f8mi_gemm_nt_kb_ws",
     "f8mi_amax_scale",
     "f8mi_amax_scale_multi",
     "f8mi_amax_tile_elems",
@@ -94,6 +96,10 @@ def lib() -> C.CDLL:
         L.f8mi_gemm_kb_ex.argtypes = [vp, i32, i32, vp, i32, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_nt.restype = i32
         L.f8mi_gemm_nt.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
+        L.f8mi_gemm_nt_ws.restype = i32
+        L.f8mi_gemm_nt_ws.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp, i64, vp]
+        L.f8mi_gemm_nt_kb_ws.restype = i32
+        L.f8mi_gemm_nt_kb_ws.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp, i64, vp]
         L.f8mi_sync.restype = i32
         L.f8mi_sync.argtypes = [vp, i32, i32, i32, i32, vp]
         L.f8mi_delayed_init.restype = i32
@@ -164,6 +170,24 @@ def workspace(dev: torch.device) -> torch.Tensor:
         ws = torch.zeros(lib().f8mi_workspace_bytes() // 4, dtype=torch.int32, device=dev)
         _workspaces[key] = ws
     return ws
+
+
+GEMM_WORKSPACE_BYTES = 32 << 20  # F8MI_GEMM_WORKSPACE_BYTES
+_GEMM_WS_MIN_ROWS, _GEMM_WS_MIN_K = 17, 2048  # below these no GEMM is ever split over k
+_gemm_workspaces = {}
+
+
+def gemm_workspace(dev: torch.device, m: int, k: int):
+    """(pointer, bytes) of the scratch that lets a few-row GEMM with a long contraction split k over workgroups; one
+    allocation per (device, stream), made the first time a shape that could use it comes by; (None, 0) for shapes
+    that never do."""
+    if m < _GEMM_WS_MIN_ROWS or k < _GEMM_WS_MIN_K:
+        return None, 0
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _raw_stream(dev))
+    ws = _gemm_workspaces.get(key)
+    if ws is None:
+        ws = _gemm_workspaces[key] = torch.empty(GEMM_WORKSPACE_BYTES // 4, dtype=torch.float32, device=dev)
+    return ws.data_ptr(), GEMM_WORKSPACE_BYTES
 
 
 def _as_2d(x: torch.Tensor) -> Tuple[torch.Tensor, int, int, int]:
@@ -342,10 +366,11 @@ def cast_dynamic(x: torch.Tensor, float8_dtype: torch.dtype, want_out: bool = Tr
 
 
 def gemm_nt_kb(a_kb: torch.Tensor, a_scale: torch.Tensor, bt_kb: torch.Tensor, b_scale: torch.Tensor,
-               out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+               out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+               split_k: bool = True) -> torch.Tensor:
     """gemm_nt on k-blocked operands: ``a_kb`` fp8 [k/64, m, 64], ``bt_kb`` fp8 [k/64, n, 64], both contiguous.
 
-    Same result bits as gemm_nt on the row-major operands.  See f8mi_gemm_nt_kb.
+    Same result bits as gemm_nt on the row-major operands (with the same ``split_k``).  See f8mi_gemm_nt_kb_ws.
     """
     _require_gpu(a_kb, "a_kb")
     _require_gpu(bt_kb, "bt_kb")
@@ -363,10 +388,11 @@ def gemm_nt_kb(a_kb: torch.Tensor, a_scale: torch.Tensor, bt_kb: torch.Tensor, b
     if bias is not None:
         assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a_kb.device
     _check_device(a_kb.device)
-    rc = lib().f8mi_gemm_nt_kb(a_kb.data_ptr(), _F8[a_kb.dtype], bt_kb.data_ptr(), _F8[bt_kb.dtype], m, n, k,
-                               a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
-                               bias.data_ptr() if bias is not None else None, _stream(a_kb))
-    _check(rc, "f8mi_gemm_nt_kb")
+    ws, ws_bytes = gemm_workspace(a_kb.device, m, k) if split_k else (None, 0)
+    rc = lib().f8mi_gemm_nt_kb_ws(a_kb.data_ptr(), _F8[a_kb.dtype], bt_kb.data_ptr(), _F8[bt_kb.dtype], m, n, k,
+                                  a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
+                                  bias.data_ptr() if bias is not None else None, ws, ws_bytes, _stream(a_kb))
+    _check(rc, "f8mi_gemm_nt_kb_ws")
     return out
 
 
@@ -397,11 +423,12 @@ def gemm_kb_ex(a_kb: torch.Tensor, a_transposed: bool, a_scale: torch.Tensor, bt
 
 
 def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: torch.Tensor, out_dtype: torch.dtype,
-            bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+            bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, split_k: bool = True) -> torch.Tensor:
     """out[m, n] = (a[m, :] . bt[n, :]) / (a_scale * b_scale) (+ bias[n]).
 
-    ``a`` is fp8 [m, k], ``bt`` is fp8 [n, k]; both must have unit stride along k.
-    See f8mi_gemm_nt.
+    ``a`` is fp8 [m, k], ``bt`` is fp8 [n, k]; both must have unit stride along k.  ``split_k``: hand the library
+    this stream's scratch buffer, with which it may split a long contraction of a few-row product over workgroups
+    (deterministic, but another summation order than without).  See f8mi_gemm_nt_ws.
     """
     _require_gpu(a, "a")
     _require_gpu(bt, "bt")
@@ -429,10 +456,11 @@ def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: t
     if bias is not None:
         assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a.device
     _check_device(a.device)
-    rc = lib().f8mi_gemm_nt(a.data_ptr(), _F8[a.dtype], lda, bt.data_ptr(), _F8[bt.dtype], ldb, m, n, k,
-                            a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
-                            bias.data_ptr() if bias is not None else None, _stream(a))
-    _check(rc, "f8mi_gemm_nt")
+    ws, ws_bytes = gemm_workspace(a.device, m, k) if split_k else (None, 0)
+    rc = lib().f8mi_gemm_nt_ws(a.data_ptr(), _F8[a.dtype], lda, bt.data_ptr(), _F8[bt.dtype], ldb, m, n, k,
+                               a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
+                               bias.data_ptr() if bias is not None else None, ws, ws_bytes, _stream(a))
+    _check(rc, "f8mi_gemm_nt_ws")
     return out
 
 

@@ -309,6 +309,13 @@ static RowSplit split_last_round(int64_t tiles_m, int64_t tiles_n, int64_t k) {
 extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fmt, int64_t ldb, int64_t m,
                             int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c,
                             int c_dtype, int64_t ldc, const void* bias_dev, void* stream_) {
+    return f8mi_gemm_nt_ws(a, a_fmt, lda, bt, b_fmt, ldb, m, n, k, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, nullptr, 0, stream_);
+}
+
+extern "C" int f8mi_gemm_nt_ws(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fmt, int64_t ldb, int64_t m,
+                               int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c,
+                               int c_dtype, int64_t ldc, const void* bias_dev, void* workspace, int64_t workspace_bytes,
+                               void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (m < 0 || n < 0 || k < 0 || lda < k || ldb < k || ldc < n) { set_error("f8mi_gemm_nt: bad shape m=%lld n=%lld k=%lld lda=%lld ldb=%lld ldc=%lld", (long long)m, (long long)n, (long long)k, (long long)lda, (long long)ldb, (long long)ldc); return F8MI_ERR_INVALID_ARG; }
     if (a_fmt < 0 || a_fmt > 1 || b_fmt < 0 || b_fmt > 1 || c_dtype < 0 || c_dtype > 2) { set_error("f8mi_gemm_nt: unknown format/dtype code"); return F8MI_ERR_INVALID_ARG; }
@@ -328,13 +335,17 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
     const uint8_t* B = (const uint8_t*)bt;
     const int M = (int)m, N = (int)n, K = (int)k;
     // Which kernel (the k-blocked entry point below decides the same way, so both give the same bits):
-    //   aligned, K % 128 == 0:  up to 16 rows, or up to 256 and a narrow Bt (use_skinny)
+    //   aligned, K % 128 == 0:  few 128-row tiles, a long k and a workspace (pick_k_splits) -> those tiles with k split over workgroups
+    //                           up to 16 rows, or up to 256 and a narrow Bt (use_skinny)
     //                                                     -> few-row kernel (Bt streamed once per 128 rows, k split over waves)
     //                           up to 256 tiles of 128 x 128 / 128 x 256 -> those
     //                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA (the tile rows of a
     //                                                        sparse last round: 128-row tiles, see split_last_round)
     //   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
     //   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
+    if (const int ks = (aligned && gemm_impl() == 0 && workspace && (uintptr_t)workspace % 16 == 0) ? pick_k_splits(M, N, K, workspace_bytes) : 0)
+        return launch_gemm_mid_splitk(a_fmt, b_fmt, c_dtype, use_mid_tiles(M, N, K) == 2, ks, (float*)workspace, stream, A, lda, 64, B, ldb, 64, M, N, K,
+                                      scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
     if (aligned && use_skinny(M, N, K) && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
     if (const int mid = (aligned && gemm_impl() == 0) ? use_mid_tiles(M, N, K) : 0)
@@ -363,6 +374,12 @@ extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* b
 extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t m, int64_t n, int64_t k,
                                const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
                                const void* bias_dev, void* stream_) {
+    return f8mi_gemm_nt_kb_ws(a, a_fmt, bt, b_fmt, m, n, k, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, nullptr, 0, stream_);
+}
+
+extern "C" int f8mi_gemm_nt_kb_ws(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t m, int64_t n, int64_t k,
+                                  const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
+                                  const void* bias_dev, void* workspace, int64_t workspace_bytes, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (m < 0 || n < 0 || k < 0 || ldc < n) { set_error("f8mi_gemm_nt_kb: bad shape m=%lld n=%lld k=%lld ldc=%lld", (long long)m, (long long)n, (long long)k, (long long)ldc); return F8MI_ERR_INVALID_ARG; }
     if (a_fmt < 0 || a_fmt > 1 || b_fmt < 0 || b_fmt > 1 || c_dtype < 0 || c_dtype > 2) { set_error("f8mi_gemm_nt_kb: unknown format/dtype code"); return F8MI_ERR_INVALID_ARG; }
@@ -377,6 +394,9 @@ extern "C" int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_f
     const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
+    if (const int ks = (gemm_impl() == 0 && workspace && (uintptr_t)workspace % 16 == 0) ? pick_k_splits(m, n, k, workspace_bytes) : 0)
+        return launch_gemm_mid_splitk(a_fmt, b_fmt, c_dtype, use_mid_tiles(m, n, k) == 2, ks, (float*)workspace, stream, (const uint8_t*)a, 64, m * 64,
+                                      (const uint8_t*)bt, 64, n * 64, (int)m, (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
     if (use_skinny(m, n, k) && gemm_impl() == 0)
         return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n,
                                   (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev);

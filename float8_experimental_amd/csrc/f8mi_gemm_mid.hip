@@ -45,7 +45,7 @@ template <int AF, int BF, int C_DT, int TJ>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
     const uint8_t* __restrict__ A, int64_t lda, int64_t a_unit, const uint8_t* __restrict__ Bt, int64_t ldb, int64_t b_unit,
     int M, int N, int K, const float* __restrict__ sa_dev, const float* __restrict__ sb_dev, void* __restrict__ C,
-    int64_t ldc, const void* __restrict__ bias, int tiles_m, int c_vec_ok) {
+    int64_t ldc, const void* __restrict__ bias, int tiles_m, int c_vec_ok, int k_splits) {
     using Cfg = MidCfg<TJ>;
     extern __shared__ __align__(16) uint8_t smem[];
     // consecutive workgroup ids go to the 8 XCDs round-robin; re-deal them so that one XCD (one L2) gets a
@@ -55,7 +55,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
     const int tm = lid % tiles_m, tn = lid / tiles_m;
     const int m0 = tm * MID_TILE_M, n0 = tn * Cfg::TILE_N;
     // 1 / (sa * sb) for the epilogue, fetched before the main loop and kept in a scalar register
-    const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
+    // k_splits > 1 (host: fp32 output, no bias): blockIdx.y takes the y-th part of k and writes its partial sums,
+    // unscaled, to the y-th M x ldc slab of C; a second kernel adds the slabs in a fixed order.
+    const int split = blockIdx.y;
+    const int K_part = K / k_splits;
+    const float inv = k_splits > 1 ? 1.0f : __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
         int, __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev))));
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -73,8 +77,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
 #pragma unroll
     for (int i = 0; i < Cfg::BI; i++)
         b_voff[i] = (uint32_t)(min((wave * Cfg::BI + i) * 16 + (lane >> 2), N - 1 - n0) * ldb) + piece;
-    const uint8_t* a_ptr = A + (int64_t)m0 * lda;
-    const uint8_t* b_ptr = Bt + (int64_t)n0 * ldb;
+    const uint8_t* a_ptr = A + (int64_t)m0 * lda + (int64_t)split * (K_part / 64) * a_unit;
+    const uint8_t* b_ptr = Bt + (int64_t)n0 * ldb + (int64_t)split * (K_part / 64) * b_unit;
     // DMA d = 0..NDMA-1 of this wave's share of a step (4 of A, then Bt); the pointers move on after the last
     auto issue1 = [&](int stage, int d) __attribute__((always_inline)) {
         const uint32_t base = lds_u32 + stage * Cfg::STAGE;
@@ -105,7 +109,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
 #pragma unroll
         for (int ti = 0; ti < 4; ti++) acc[tj][ti] = (v4f_m){0.f, 0.f, 0.f, 0.f};
 
-    const int steps = K / 128;
+    const int steps = K_part / 128;
     constexpr int LEAD = Cfg::NSTAGE - 1;  // steps of data in flight
 #pragma unroll
     for (int p = 0; p < LEAD; p++)
@@ -179,7 +183,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = acc[tj][ti][e] * inv + bv[e];
-                float* dst = (float*)C + (int64_t)row * ldc + col;
+                float* dst = (float*)C + ((int64_t)split * M + row) * ldc + col;
                 if (c_vec_ok && col + 4 <= N) {
                     *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
                 } else {
@@ -236,41 +240,102 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
 template <int AF, int BF, int C_DT, int TJ>
 static int launch_mid4(hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb,
                        int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
-                       int c_vec_ok) {
+                       int c_vec_ok, int k_splits) {
     static std::atomic<uint64_t> lds_allowed{0};
     auto kern = gemm_mid_kernel<AF, BF, C_DT, TJ>;
     if (int rc = allow_big_lds(kern, MidCfg<TJ>::LDS, lds_allowed)) return rc;
     const int tiles_m = (M + MID_TILE_M - 1) / MID_TILE_M, tiles_n = (N + MidCfg<TJ>::TILE_N - 1) / MidCfg<TJ>::TILE_N;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(GEMM_THREADS), MidCfg<TJ>::LDS, stream, A, lda, a_unit, Bt, ldb, b_unit,
-                       M, N, K, sa, sb, C, ldc, bias, tiles_m, c_vec_ok);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)k_splits), dim3(GEMM_THREADS), MidCfg<TJ>::LDS, stream, A, lda, a_unit,
+                       Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, tiles_m, c_vec_ok, k_splits);
     return check_hip(hipGetLastError(), "gemm (128-row tiles) kernel launch");
 }
 
 template <int AF, int BF, int C_DT>
 static int launch_mid3(bool wide, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb,
                        int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc, const void* bias,
-                       int c_vec_ok) {
-    if (wide) return launch_mid4<AF, BF, C_DT, 8>(stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
-    return launch_mid4<AF, BF, C_DT, 4>(stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
+                       int c_vec_ok, int k_splits) {
+    if (wide) return launch_mid4<AF, BF, C_DT, 8>(stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
+    return launch_mid4<AF, BF, C_DT, 4>(stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
 }
 
 template <int AF, int BF>
 static int launch_mid2(int c_dtype, bool wide, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit, const uint8_t* Bt,
                        int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C, int64_t ldc,
-                       const void* bias, int c_vec_ok) {
-    if (c_dtype == F8MI_BF16) return launch_mid3<AF, BF, F8MI_BF16>(wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
-    if (c_dtype == F8MI_FP16) return launch_mid3<AF, BF, F8MI_FP16>(wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
-    return launch_mid3<AF, BF, F8MI_FP32>(wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
+                       const void* bias, int c_vec_ok, int k_splits) {
+    if (c_dtype == F8MI_BF16) return launch_mid3<AF, BF, F8MI_BF16>(wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
+    if (c_dtype == F8MI_FP16) return launch_mid3<AF, BF, F8MI_FP16>(wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
+    return launch_mid3<AF, BF, F8MI_FP32>(wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
+}
+
+static int launch_mid1(int a_fmt, int b_fmt, int c_dtype, bool wide, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
+                       const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
+                       int64_t ldc, const void* bias, int c_vec_ok, int k_splits) {
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_mid2<0, 0>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
+    if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_mid2<1, 0>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
+    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_mid2<0, 1>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
+    return launch_mid2<1, 1>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, k_splits);
 }
 
 // wide: 128 x 256 tiles instead of 128 x 128
 int launch_gemm_mid(int a_fmt, int b_fmt, int c_dtype, bool wide, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                     const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                     int64_t ldc, const void* bias, int c_vec_ok) {
-    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_mid2<0, 0>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
-    if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_mid2<1, 0>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
-    if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E5M2) return launch_mid2<0, 1>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
-    return launch_mid2<1, 1>(c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok);
+    return launch_mid1(a_fmt, b_fmt, c_dtype, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, C, ldc, bias, c_vec_ok, 1);
+}
+
+// C = (partial[0] + partial[1] + ... in this order) / (sa * sb) + bias: four neighbouring columns per lane (N % 4 == 0)
+template <int C_DT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int k_splits, int M, int N,
+                                                            const float* __restrict__ sa_dev, const float* __restrict__ sb_dev,
+                                                            void* __restrict__ C, int64_t ldc, const void* __restrict__ bias, int c_vec_ok) {
+    const int64_t quads = (int64_t)N / 4;
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= (int64_t)M * quads) return;
+    const int64_t row = q / quads;
+    const int col = (int)(q % quads) * 4;
+    const float inv = __fdiv_rn(1.0f, *sa_dev) * __fdiv_rn(1.0f, *sb_dev);
+    const int64_t slab = (int64_t)M * N;
+    float4 sum = *(const float4*)(partial + row * N + col);
+    for (int s = 1; s < k_splits; s++) {
+        const float4 p = *(const float4*)(partial + s * slab + row * N + col);
+        sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+    }
+    float v[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = v[e] * inv + (bias ? load_bias<C_DT>(bias, col + e) : 0.f);
+    if constexpr (C_DT == F8MI_FP32) {
+        float* dst = (float*)C + row * ldc + col;
+        if (c_vec_ok) {
+            *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) dst[e] = v[e];
+        }
+    } else {
+        uint16_t* dst = (uint16_t*)C + row * ldc + col;
+        const uint32_t p0 = pack2<C_DT>(v[0], v[1]), p1 = pack2<C_DT>(v[2], v[3]);
+        if (c_vec_ok) {  // rows start 16-byte aligned, col % 4 == 0: 8-byte aligned
+            *(uint2*)dst = make_uint2(p0, p1);
+        } else {
+            dst[0] = (uint16_t)(p0 & 0xffffu); dst[1] = (uint16_t)(p0 >> 16);
+            dst[2] = (uint16_t)(p1 & 0xffffu); dst[3] = (uint16_t)(p1 >> 16);
+        }
+    }
+}
+
+// The contraction split k_splits ways over workgroups (outputs of few tiles and a long k: every CU gets a part).
+// `partial` holds k_splits x M x N floats (16-byte aligned); host side has checked K % (128 * k_splits) == 0, N % 4 == 0.
+int launch_gemm_mid_splitk(int a_fmt, int b_fmt, int c_dtype, bool wide, int k_splits, float* partial, hipStream_t stream, const uint8_t* A,
+                           int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa,
+                           const float* sb, void* C, int64_t ldc, const void* bias, int c_vec_ok) {
+    if (int rc = launch_mid1(a_fmt, b_fmt, F8MI_FP32, wide, stream, A, lda, a_unit, Bt, ldb, b_unit, M, N, K, sa, sb, partial, N, nullptr, 1, k_splits))
+        return rc;
+    const int64_t quads = (int64_t)M * (N / 4);
+    const dim3 grid((unsigned)((quads + 255) / 256));
+    if (c_dtype == F8MI_BF16) hipLaunchKernelGGL(splitk_reduce_kernel<F8MI_BF16>, grid, dim3(256), 0, stream, partial, k_splits, M, N, sa, sb, C, ldc, bias, c_vec_ok);
+    else if (c_dtype == F8MI_FP16) hipLaunchKernelGGL(splitk_reduce_kernel<F8MI_FP16>, grid, dim3(256), 0, stream, partial, k_splits, M, N, sa, sb, C, ldc, bias, c_vec_ok);
+    else hipLaunchKernelGGL(splitk_reduce_kernel<F8MI_FP32>, grid, dim3(256), 0, stream, partial, k_splits, M, N, sa, sb, C, ldc, bias, c_vec_ok);
+    return check_hip(hipGetLastError(), "gemm split-k reduction kernel launch");
 }
 
 }  // namespace f8mi

@@ -186,27 +186,58 @@ inline int use_mid_tiles(int64_t m, int64_t n, int64_t k) {
 }
 // few-row kernel (f8mi_gemm_skinny.hip): m <= SKINNY_MAX_M, K % 128 == 0, aligned operands.
 constexpr int SKINNY_MAX_M = 256;
-// Up to 16 rows the few-row kernel always runs: it streams Bt once at memory speed.  With more rows every one of its
-// 32-column workgroups re-reads A from L2, and from 129 rows on it passes over Bt twice, so a wide Bt is cheaper
-// as one round (or two) of 128-row tiles, which take the same time for 1 or 128 rows.  Estimates in us, fitted to
-// measurements (rows, n x k: few-row / tiles): 128, 8192 x 8192: 27 / 37; 128, 28672 x 8192: 83 / 37; 64, 28672 x 8192:
-// 53 / 37; 144 - 256, 4096 x 4096: 14 / 20; 4096 x 14336: 36 / 60; 8192 x 8192: 41 - 48 / 37; 14336 x 4096: 39 - 47 / 22;
-// 28672 x 8192: 119 - 143 / 59.  Depends on the shape only, so the row-major and the k-blocked entry point agree.
+// Time estimates in us behind the choice between the few-row kernel, a round of 128-row tiles, and the same tiles
+// with k split over workgroups -- fitted to measurements (rows, n x k: few-row / tiles): 128, 8192 x 8192: 27 / 37;
+// 128, 28672 x 8192: 83 / 37; 64, 28672 x 8192: 53 / 37; 64, 4096 x 14336: 27 / 63; 144 - 256, 4096 x 4096: 14 / 20;
+// 4096 x 14336: 36 / 60; 8192 x 8192: 41 - 48 / 37; 14336 x 4096: 39 - 47 / 22; 28672 x 8192: 119 - 143 / 59.
+// They depend on the shape only, so the row-major and the k-blocked entry point decide alike.
+//
+// Few-row kernel: Bt at 6.5 TB/s from memory plus A (n / 32 workgroups x 16 row_tiles x k bytes) at 20 TB/s from L2,
+// once per 128 rows; slower when its n / 32 workgroups per pass leave CUs idle.
+inline double skinny_time_us(int64_t m, int64_t n, int64_t k) {
+    const double passes = (double)((m + 127) / 128);
+    const double row_tiles = m > 128 ? 8.0 : (double)((m + 15) / 16);  // 16-row tiles of A per pass
+    const double wgs = passes * (double)((n + 31) / 32);
+    const double idle = wgs < 256.0 ? __builtin_sqrt(256.0 / wgs) : 1.0;
+    return passes * (2.0 + (double)n * (double)k * (0.154 + 0.025 * row_tiles) * 1e-6 * idle);
+}
+// Tiles: a round of 128 x 128 tiles takes 4.4 ns per unit of k, of 128 x 256 tiles 7.8 ns, of 256 x 256 tiles 10.6 ns,
+// for 1 row or 128.
+inline double tiles_time_us(int64_t m, int64_t n, int64_t k) {
+    const int64_t rt = (m + 127) / 128;
+    if (rt * ((n + 127) / 128) <= 256) return 4.4e-3 * (double)k;
+    if (rt * ((n + 255) / 256) <= 256) return 7.8e-3 * (double)k;
+    return 10.6e-3 * (double)k * (double)((((m + 255) / 256) * ((n + 255) / 256) + 255) / 256);
+}
+// Up to 16 rows the few-row kernel always runs: it streams Bt once at memory speed.
 inline bool use_skinny(int64_t m, int64_t n, int64_t k) {
     if (m > SKINNY_MAX_M || k <= 0 || k % 128 != 0) return false;
     if (m <= 16) return true;
-    const double passes = (double)((m + 127) / 128);
-    const double row_tiles = m > 128 ? 8.0 : (double)((m + 15) / 16);  // 16-row tiles of A per pass
-    // Bt at 6.5 TB/s from memory plus A (n / 32 workgroups x 16 row_tiles x k bytes) at 20 TB/s from L2
-    const double t_skinny = passes * (2.0 + (double)n * (double)k * (0.154 + 0.025 * row_tiles) * 1e-6);
-    // one round of 128 x 128 tiles: 4.4 ns per unit of k; of 128 x 256 tiles: 7.8 ns; of 256 x 256 tiles: 10.6 ns
-    const int64_t rt = (m + 127) / 128;
-    double t_tiles;
-    if (rt * ((n + 127) / 128) <= 256) t_tiles = 4.4e-3 * (double)k;
-    else if (rt * ((n + 255) / 256) <= 256) t_tiles = 7.8e-3 * (double)k;
-    else t_tiles = 10.6e-3 * (double)k * (double)((((m + 255) / 256) * ((n + 255) / 256) + 255) / 256);
-    return t_skinny <= t_tiles;
+    return skinny_time_us(m, n, k) <= tiles_time_us(m, n, k);
 }
+// An output of at most 128 of the 128-row tiles and a long k: with `ws_bytes` of scratch for the partial sums, k is
+// split 2, 4 or 8 ways so that (nearly) every CU gets a part, and a second kernel adds the parts in a fixed order.
+// Returns the number of parts, 0 for no split.  Cost of the split: the parts written and read once (5 TB/s) and a launch.
+inline int pick_k_splits(int64_t m, int64_t n, int64_t k, int64_t ws_bytes) {
+    const int mode = use_mid_tiles(m, n, k);
+    if (!mode || n % 4 != 0 || m <= 16 || ws_bytes <= 0) return 0;
+    const int64_t tiles = ((m + 127) / 128) * ((n + (mode == 1 ? 127 : 255)) / (mode == 1 ? 128 : 256));
+    if (tiles > 128) return 0;
+    const double t_round = (mode == 1 ? 4.4e-3 : 7.8e-3) * (double)k;
+    const double t_skinny = m <= SKINNY_MAX_M ? skinny_time_us(m, n, k) : 1e30;
+    const double t_other = t_skinny < t_round ? t_skinny : t_round;
+    int best = 0;
+    double t_best = 0.9 * t_other;  // the estimates are not better than that
+    for (int s = 2; s <= 8; s *= 2) {
+        if (tiles * s > 256 || k % (128 * s) != 0 || k / s < 1024 || (int64_t)s * m * n * 4 > ws_bytes) break;
+        const double t = t_round / s + 3.0 + (double)s * (double)m * (double)n * 8.0 / 5e6 + 4.0;
+        if (t < t_best) { t_best = t; best = s; }
+    }
+    return best;
+}
+int launch_gemm_mid_splitk(int a_fmt, int b_fmt, int c_dtype, bool wide, int k_splits, float* partial, hipStream_t stream, const uint8_t* A,
+                           int64_t lda, int64_t a_unit, const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa,
+                           const float* sb, void* C, int64_t ldc, const void* bias, int c_vec_ok);
 int launch_gemm_skinny(int a_fmt, int b_fmt, int c_dtype, hipStream_t stream, const uint8_t* A, int64_t lda, int64_t a_unit,
                        const uint8_t* Bt, int64_t ldb, int64_t b_unit, int M, int N, int K, const float* sa, const float* sb, void* C,
                        int64_t ldc, const void* bias);

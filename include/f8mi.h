@@ -182,6 +182,23 @@ int f8mi_gemm_nt_kb(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t
                     const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
                     const void* bias_dev, void* stream);
 
+/* f8mi_gemm_nt / f8mi_gemm_nt_kb with scratch memory for the library to use: `workspace` (16-byte aligned device
+ * memory, `workspace_bytes` long, contents irrelevant before and after; calls sharing it must not overlap) lets an
+ * output of few tiles with a long k be computed with k split over workgroups -- an inference linear with 17 to a few
+ * hundred rows and a long contraction, which would otherwise leave most CUs idle: partial sums go to the workspace
+ * and a second kernel adds them in a fixed order (deterministic; another summation order than without the split,
+ * so the two agree within the accumulation tolerance, not bit for bit).  Which path runs depends on (m, n, k),
+ * alignment and workspace_bytes only; F8MI_GEMM_WORKSPACE_BYTES is enough for every case that is ever split.
+ * With workspace NULL they are f8mi_gemm_nt / f8mi_gemm_nt_kb.  No counterpart in the reference (torch._scaled_mm
+ * hides hipBLASLt's own workspace, float8_python_api.py:24-64). */
+#define F8MI_GEMM_WORKSPACE_BYTES (32ll << 20)
+int f8mi_gemm_nt_ws(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fmt, int64_t ldb, int64_t m,
+                    int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
+                    int64_t ldc, const void* bias_dev, void* workspace, int64_t workspace_bytes, void* stream);
+int f8mi_gemm_nt_kb_ws(const void* a, int a_fmt, const void* bt, int b_fmt, int64_t m, int64_t n, int64_t k,
+                       const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
+                       const void* bias_dev, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* f8mi_gemm_nt_kb with operands that may be given transposed, so that one k-blocked copy of a tensor serves
  * both GEMMs that use it (no transposed fp8 copies at all):
  *   a, a_transposed = 0: [k/64][m][64] as above;  = 1: [m/64][k][64], i.e. the matrix [k][m] k-blocked over m

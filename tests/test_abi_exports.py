@@ -56,6 +56,11 @@ def test_host_side_argument_checks_need_no_gpu():
     # k-blocked operands: k must be a multiple of 64 and at least 384 (unsupported, not invalid)
     rc = lib.f8mi_gemm_nt_kb(None, 0, None, 0, i64(4), i64(4), i64(100), None, None, None, 0, i64(4), None, None)
     assert rc == -2 and b"k-blocked" in lib.f8mi_last_error()
+    # the workspace variants check their arguments like the plain ones
+    rc = lib.f8mi_gemm_nt_kb_ws(None, 0, None, 0, i64(4), i64(4), i64(100), None, None, None, 0, i64(4), None, None, i64(0), None)
+    assert rc == -2 and b"k-blocked" in lib.f8mi_last_error()
+    rc = lib.f8mi_gemm_nt_ws(None, 0, i64(8), None, 0, i64(8), i64(-1), i64(4), i64(8), None, None, None, 0, i64(4), None, None, i64(0), None)
+    assert rc == -1
     # transposed operands: (a transposed, bt not) is not built; row counts must be multiples of 64
     rc = lib.f8mi_gemm_kb_ex(None, 0, 1, None, 0, 0, i64(64), i64(64), i64(384), None, None, None, 0, i64(64), None, None)
     assert rc == -2

@@ -440,6 +440,30 @@ def test_gemm_mid_tile_kernel_shapes(nat, m, n, k, out_dt):
     _gemm_check(nat, m, n, k, fm[0], fm[1], out_dt, seed=m + n + k, bias=(n % 2 == 0))
 
 
+# Few 128-row tiles and a long contraction: with the stream's scratch buffer k is split over workgroups and a second
+# kernel adds the parts in a fixed order.
+@pytest.mark.parametrize("m,n,k", [(256, 2048, 16384), (512, 1024, 8192), (100, 4096, 16384)])
+def test_gemm_split_over_k(nat, m, n, k):
+    a = _rand_fp8((m, k), torch.float8_e4m3fn, m + k, 4.0).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e5m2, n + k, 4.0).to(DEV)
+    sa, sb = torch.tensor(0.5, device=DEV), torch.tensor(4.0, device=DEV)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 3).to(torch.bfloat16).to(DEV)
+    split32 = nat.gemm_nt(a, sa, bt, sb, torch.float32)
+    whole32 = nat.gemm_nt(a, sa, bt, sb, torch.float32, split_k=False)
+    # another summation order (else the split did not run) but the same sums to fp32 accuracy, every time the same bits,
+    # whichever layout the operands come in
+    assert not torch.equal(split32, whole32)
+    scale = whole32.abs().max()
+    assert ((split32 - whole32).abs().max() / scale).item() < 1e-5
+    assert torch.equal(nat.gemm_nt(a, sa, bt, sb, torch.float32), split32)
+    assert torch.equal(nat.gemm_nt_kb(_to_kb(a), sa, _to_kb(bt), sb, torch.float32), split32)
+    got = nat.gemm_nt_kb(_to_kb(a), sa, _to_kb(bt), sb, torch.bfloat16, bias=bias)
+    assert torch.equal(got, nat.gemm_nt(a, sa, bt, sb, torch.bfloat16, bias=bias))
+    want = (split32 + bias.float()).to(torch.bfloat16)  # one rounding of the scaled sum plus bias
+    assert ((got.float() - want.float()).abs() <= 2 * torch.finfo(torch.bfloat16).eps * want.float().abs() + 1e-6).all()
+    _gemm_check(nat, m, n, k, "e4m3", "e5m2", torch.bfloat16, seed=m + n, bias=True)
+
+
 # More than one round of 256 x 256 tiles with few tiles in the last one: the last tile rows go to a 128-row-tile kernel.
 @pytest.mark.parametrize("m,n,k,m_pad", [(4352, 4096, 512, 8192),      # 272 tiles: 16 of them as 128 x 128 tiles
                                          (8500, 2048, 384, 16384),     # ragged last tile row
@@ -571,7 +595,7 @@ def test_gemm_with_transposed_operands_equals_row_major_bitwise(nat, m, n, k):
     # another order: pad A with zero rows past that limit and cut the result)
     a_ref = a if m > 256 else torch.cat([a.view(torch.uint8), torch.zeros(320 - m, k, dtype=torch.uint8, device=DEV)]).view(a.dtype)
     for out_dt, b in ((torch.bfloat16, bias), (torch.float32, None)):
-        want = nat.gemm_nt(a_ref, sa, bt, sb, out_dt, bias=b)[:m]
+        want = nat.gemm_nt(a_ref, sa, bt, sb, out_dt, bias=b, split_k=False)[:m]  # transposed operands are never split over k
         got = nat.gemm_kb_ex(_to_kb(a), False, sa, bt_tr, True, sb, out_dt, bias=b)
         assert torch.equal(got, want), (m, n, k, out_dt, "bt transposed")
         got = nat.gemm_kb_ex(a_tr, True, sa, bt_tr, True, sb, out_dt, bias=b)
