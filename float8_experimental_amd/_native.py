@@ -30,6 +30,7 @@ EXPORTS = (
     "f8mi_workspace_bytes",
     "f8mi_gemm_nt_ws",
     "f8mi_gemm_nt_kb_ws",
+    "f8mi_gemm_plan",
     "f8mi_amax_scale",
     "f8mi_amax_scale_multi",
     "f8mi_amax_tile_elems",
@@ -98,6 +99,8 @@ def lib() -> C.CDLL:
         L.f8mi_gemm_nt.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_nt_ws.restype = i32
         L.f8mi_gemm_nt_ws.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp, i64, vp]
+        L.f8mi_gemm_plan.restype = i32
+        L.f8mi_gemm_plan.argtypes = [i64, i64, i64, i32, i64]
         L.f8mi_gemm_nt_kb_ws.restype = i32
         L.f8mi_gemm_nt_kb_ws.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp, i64, vp]
         L.f8mi_sync.restype = i32
@@ -188,6 +191,18 @@ def gemm_workspace(dev: torch.device, m: int, k: int):
     if ws is None:
         ws = _gemm_workspaces[key] = torch.empty(GEMM_WORKSPACE_BYTES // 4, dtype=torch.float32, device=dev)
     return ws.data_ptr(), GEMM_WORKSPACE_BYTES
+
+
+PLAN_NAMES = {1: "tiles128_split_k", 2: "few_rows", 3: "tiles128", 4: "tiles256", 5: "tiles256_and_128", 6: "tiles256_mfma32",
+              7: "staged"}
+
+
+def gemm_plan(m: int, n: int, k: int, aligned: bool = True, split_k: bool = True):
+    """(kernel name, parts of k, 0 / 1 / 2 for none / 128 x 128 / 128 x 256 tiles) the library picks for an m x n x k
+    product, as gemm_nt / gemm_nt_kb call it (``split_k``: with the scratch buffer they pass).  Needs no GPU."""
+    ws = GEMM_WORKSPACE_BYTES if split_k and m >= _GEMM_WS_MIN_ROWS and k >= _GEMM_WS_MIN_K else 0
+    code = lib().f8mi_gemm_plan(m, n, k, int(aligned), ws)
+    return PLAN_NAMES.get(code & 0xff), (code >> 8) & 0xff, (code >> 16) & 0xff
 
 
 def _as_2d(x: torch.Tensor) -> Tuple[torch.Tensor, int, int, int]:

@@ -306,6 +306,48 @@ static RowSplit split_last_round(int64_t tiles_m, int64_t tiles_n, int64_t k) {
     return {rows_large, mid};
 }
 
+// Which kernel computes an m x n x k product (codes: include/f8mi.h, F8MI_PLAN_*).  One function for both entry points,
+// so that row-major and k-blocked operands of one shape always take the same kernel and give the same bits.
+//   aligned, K % 128 == 0:  few 128-row tiles, a long k and a workspace (pick_k_splits) -> those tiles with k split over workgroups
+//                           up to 16 rows, or up to 256 and a narrow Bt (use_skinny)
+//                                                     -> few-row kernel (Bt streamed once per 128 rows, k split over waves)
+//                           up to 256 tiles of 128 x 128 / 128 x 256 -> those
+//                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA (the tile rows of a
+//                                                        sparse last round: 128-row tiles, see split_last_round)
+//   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
+//   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
+// F8MI_GEMM_IMPL=staged forces the register-staged kernel, =dma32 the 32x32x64 LDS-DMA kernel (comparison runs).
+struct GemmPlan { int kind; int parts; int mid; RowSplit split; };
+static GemmPlan gemm_plan(int64_t m, int64_t n, int64_t k, bool aligned, int64_t ws_bytes) {
+    GemmPlan p{F8MI_PLAN_STAGED, 0, 0, {0, 0}};
+    const int impl = gemm_impl();
+    if (aligned && impl == 0) {
+        if (const int parts = pick_k_splits(m, n, k, ws_bytes)) {
+            p.kind = F8MI_PLAN_TILES128_SPLIT_K; p.parts = parts; p.mid = use_mid_tiles(m, n, k);
+            return p;
+        }
+        if (use_skinny(m, n, k)) { p.kind = F8MI_PLAN_FEW_ROWS; return p; }
+        if (const int mid = use_mid_tiles(m, n, k)) { p.kind = F8MI_PLAN_TILES128; p.mid = mid; return p; }
+    }
+    if (aligned && k >= 384 && k % 64 == 0 && impl != 1) {
+        if (k % 128 == 0 && impl != 2) {
+            const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+            p.split = impl == 0 ? split_last_round(tiles_m, tiles_n, k) : RowSplit{0, 0};
+            p.kind = p.split.rows_large ? F8MI_PLAN_TILES256_AND_128 : F8MI_PLAN_TILES256;
+            p.mid = p.split.mid;
+            return p;
+        }
+        p.kind = F8MI_PLAN_TILES256_MFMA32;
+    }
+    return p;
+}
+
+extern "C" int f8mi_gemm_plan(int64_t m, int64_t n, int64_t k, int aligned, int64_t workspace_bytes) {
+    if (m <= 0 || n <= 0 || k < 0) return 0;
+    const GemmPlan p = gemm_plan(m, n, k, aligned != 0, workspace_bytes);
+    return p.kind | (p.parts << 8) | (p.mid << 16);
+}
+
 extern "C" int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fmt, int64_t ldb, int64_t m,
                             int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c,
                             int c_dtype, int64_t ldc, const void* bias_dev, void* stream_) {
@@ -334,36 +376,29 @@ extern "C" int f8mi_gemm_nt_ws(const void* a, int a_fmt, int64_t lda, const void
     const uint8_t* A = (const uint8_t*)a;
     const uint8_t* B = (const uint8_t*)bt;
     const int M = (int)m, N = (int)n, K = (int)k;
-    // Which kernel (the k-blocked entry point below decides the same way, so both give the same bits):
-    //   aligned, K % 128 == 0:  few 128-row tiles, a long k and a workspace (pick_k_splits) -> those tiles with k split over workgroups
-    //                           up to 16 rows, or up to 256 and a narrow Bt (use_skinny)
-    //                                                     -> few-row kernel (Bt streamed once per 128 rows, k split over waves)
-    //                           up to 256 tiles of 128 x 128 / 128 x 256 -> those
-    //                           K >= 384                  -> 256 x 256 tiles, 16x16x128 MFMA, LDS-DMA (the tile rows of a
-    //                                                        sparse last round: 128-row tiles, see split_last_round)
-    //   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
-    //   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
-    if (const int ks = (aligned && gemm_impl() == 0 && workspace && (uintptr_t)workspace % 16 == 0) ? pick_k_splits(M, N, K, workspace_bytes) : 0)
-        return launch_gemm_mid_splitk(a_fmt, b_fmt, c_dtype, use_mid_tiles(M, N, K) == 2, ks, (float*)workspace, stream, A, lda, 64, B, ldb, 64, M, N, K,
-                                      scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
-    if (aligned && use_skinny(M, N, K) && gemm_impl() == 0)
-        return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
-    if (const int mid = (aligned && gemm_impl() == 0) ? use_mid_tiles(M, N, K) : 0)
-        return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
-    // F8MI_GEMM_IMPL=staged forces the register-staged kernel, =dma32 the 32x32x64 LDS-DMA kernel (comparison runs)
-    if (aligned && K >= 384 && K % 64 == 0 && gemm_impl() != 1) {
-        if (K % 128 == 0 && gemm_impl() != 2) {
-            if (const RowSplit sp = gemm_impl() == 0 ? split_last_round(tiles_m, tiles_n, K) : RowSplit{0, 0}; sp.rows_large) {
-                const int m1 = (int)(sp.rows_large * BM);
-                if (int rc = launch_gemm_dma16(a_fmt, b_fmt, c_dtype, dim3((unsigned)(sp.rows_large * tiles_n)), stream, A, lda, 64, B, ldb, 64, m1, N, K,
-                                               scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)sp.rows_large, (int)tiles_n, c_vec_ok))
-                    return rc;
-                return launch_gemm_mid(a_fmt, b_fmt, c_dtype, sp.mid == 2, stream, A + (int64_t)m1 * lda, lda, 64, B, ldb, 64, M - m1, N, K, scale_a_dev,
-                                       scale_b_dev, (uint8_t*)c + (int64_t)m1 * ldc * csz, ldc, bias_dev, c_vec_ok);
-            }
-            return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    const bool ws_ok = workspace && (uintptr_t)workspace % 16 == 0;
+    const GemmPlan plan = gemm_plan(m, n, k, aligned, ws_ok ? workspace_bytes : 0);
+    switch (plan.kind) {
+        case F8MI_PLAN_TILES128_SPLIT_K:
+            return launch_gemm_mid_splitk(a_fmt, b_fmt, c_dtype, plan.mid == 2, plan.parts, (float*)workspace, stream, A, lda, 64, B, ldb, 64, M, N, K,
+                                          scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
+        case F8MI_PLAN_FEW_ROWS:
+            return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
+        case F8MI_PLAN_TILES128:
+            return launch_gemm_mid(a_fmt, b_fmt, c_dtype, plan.mid == 2, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
+        case F8MI_PLAN_TILES256_AND_128: {
+            const int m1 = (int)(plan.split.rows_large * BM);
+            if (int rc = launch_gemm_dma16(a_fmt, b_fmt, c_dtype, dim3((unsigned)(plan.split.rows_large * tiles_n)), stream, A, lda, 64, B, ldb, 64, m1, N, K,
+                                           scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)plan.split.rows_large, (int)tiles_n, c_vec_ok))
+                return rc;
+            return launch_gemm_mid(a_fmt, b_fmt, c_dtype, plan.mid == 2, stream, A + (int64_t)m1 * lda, lda, 64, B, ldb, 64, M - m1, N, K, scale_a_dev,
+                                   scale_b_dev, (uint8_t*)c + (int64_t)m1 * ldc * csz, ldc, bias_dev, c_vec_ok);
         }
-        return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+        case F8MI_PLAN_TILES256:
+            return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+        case F8MI_PLAN_TILES256_MFMA32:
+            return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, lda, 64, B, ldb, 64, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+        default: break;  // F8MI_PLAN_STAGED
     }
     if (a_fmt == F8MI_E4M3FN && b_fmt == F8MI_E4M3FN) return launch_gemm1<0, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
     if (a_fmt == F8MI_E5M2 && b_fmt == F8MI_E4M3FN) return launch_gemm1<1, 0>(aligned, c_dtype, g, stream, A, lda, B, ldb, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
@@ -394,31 +429,37 @@ extern "C" int f8mi_gemm_nt_kb_ws(const void* a, int a_fmt, const void* bt, int 
     const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
-    if (const int ks = (gemm_impl() == 0 && workspace && (uintptr_t)workspace % 16 == 0) ? pick_k_splits(m, n, k, workspace_bytes) : 0)
-        return launch_gemm_mid_splitk(a_fmt, b_fmt, c_dtype, use_mid_tiles(m, n, k) == 2, ks, (float*)workspace, stream, (const uint8_t*)a, 64, m * 64,
-                                      (const uint8_t*)bt, 64, n * 64, (int)m, (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
-    if (use_skinny(m, n, k) && gemm_impl() == 0)
-        return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n,
-                                  (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
-    if (const int mid = gemm_impl() == 0 ? use_mid_tiles(m, n, k) : 0)
-        return launch_gemm_mid(a_fmt, b_fmt, c_dtype, mid == 2, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m, (int)n, (int)k,
-                               scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
-    if (k % 128 == 0 && gemm_impl() != 2) {
-        if (const RowSplit sp = gemm_impl() == 0 ? split_last_round(tiles_m, tiles_n, k) : RowSplit{0, 0}; sp.rows_large) {
+    const uint8_t* A = (const uint8_t*)a;
+    const uint8_t* B = (const uint8_t*)bt;
+    const int M = (int)m, N = (int)n, K = (int)k;
+    const int64_t a_unit = m * 64, b_unit = n * 64;  // bytes between 64-deep blocks
+    const bool ws_ok = workspace && (uintptr_t)workspace % 16 == 0;
+    const GemmPlan plan = gemm_plan(m, n, k, true, ws_ok ? workspace_bytes : 0);
+    switch (plan.kind) {
+        case F8MI_PLAN_TILES128_SPLIT_K:
+            return launch_gemm_mid_splitk(a_fmt, b_fmt, c_dtype, plan.mid == 2, plan.parts, (float*)workspace, stream, A, 64, a_unit, B, 64, b_unit, M, N, K,
+                                          scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
+        case F8MI_PLAN_FEW_ROWS:
+            return launch_gemm_skinny(a_fmt, b_fmt, c_dtype, stream, A, 64, a_unit, B, 64, b_unit, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev);
+        case F8MI_PLAN_TILES128:
+            return launch_gemm_mid(a_fmt, b_fmt, c_dtype, plan.mid == 2, stream, A, 64, a_unit, B, 64, b_unit, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, c_vec_ok);
+        case F8MI_PLAN_TILES256_AND_128: {
             // rows m1 .. m of a k-blocked operand start m1 * 64 bytes in; the distance between 64-deep blocks stays m * 64
-            const int64_t m1 = sp.rows_large * BM;
-            if (int rc = launch_gemm_dma16(a_fmt, b_fmt, c_dtype, dim3((unsigned)(sp.rows_large * tiles_n)), stream, (const uint8_t*)a, 64, m * 64,
-                                           (const uint8_t*)bt, 64, n * 64, (int)m1, (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev,
-                                           (int)sp.rows_large, (int)tiles_n, c_vec_ok))
+            const int64_t m1 = plan.split.rows_large * BM;
+            if (int rc = launch_gemm_dma16(a_fmt, b_fmt, c_dtype, dim3((unsigned)(plan.split.rows_large * tiles_n)), stream, A, 64, a_unit, B, 64, b_unit,
+                                           (int)m1, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)plan.split.rows_large, (int)tiles_n, c_vec_ok))
                 return rc;
-            return launch_gemm_mid(a_fmt, b_fmt, c_dtype, sp.mid == 2, stream, (const uint8_t*)a + m1 * 64, 64, m * 64, (const uint8_t*)bt, 64, n * 64,
-                                   (int)(m - m1), (int)n, (int)k, scale_a_dev, scale_b_dev, (uint8_t*)c + m1 * ldc * csz, ldc, bias_dev, c_vec_ok);
+            return launch_gemm_mid(a_fmt, b_fmt, c_dtype, plan.mid == 2, stream, A + m1 * 64, 64, a_unit, B, 64, b_unit, (int)(m - m1), N, K, scale_a_dev,
+                                   scale_b_dev, (uint8_t*)c + m1 * ldc * csz, ldc, bias_dev, c_vec_ok);
         }
-        return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
-                                 (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+        default: break;
     }
-    return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, n * 64, (int)m,
-                           (int)n, (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    // whole output on 256 x 256 tiles (there is no register-staged kernel for k-blocked operands: F8MI_GEMM_IMPL=staged means these)
+    if (k % 128 == 0 && gemm_impl() != 2)
+        return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, A, 64, a_unit, B, 64, b_unit, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev,
+                                 (int)tiles_m, (int)tiles_n, c_vec_ok);
+    return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, 64, a_unit, B, 64, b_unit, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev,
+                           (int)tiles_m, (int)tiles_n, c_vec_ok);
 }
 
 extern "C" int f8mi_gemm_kb_ex(const void* a, int a_fmt, int a_transposed, const void* bt, int b_fmt, int b_transposed,

@@ -199,6 +199,20 @@ int f8mi_gemm_nt_kb_ws(const void* a, int a_fmt, const void* bt, int b_fmt, int6
                        const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype, int64_t ldc,
                        const void* bias_dev, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Which kernel f8mi_gemm_nt(_ws) / f8mi_gemm_nt_kb(_ws) would run for an m x n x k product (no GPU needed; for tests,
+ * logs and benchmarks).  `aligned`: operands and row strides are 16-byte aligned (k-blocked operands always are);
+ * workspace_bytes: 0 without a workspace.  Returns a F8MI_PLAN_* code in bits 0-7, the number of parts k is split
+ * into in bits 8-15 and, where 128-row tiles take part, 1 (128 x 128) or 2 (128 x 256) in bits 16-23; 0 for an
+ * empty product.  No counterpart in the reference. */
+#define F8MI_PLAN_TILES128_SPLIT_K 1 /* 128-row tiles, k split over workgroups, second kernel adds the parts */
+#define F8MI_PLAN_FEW_ROWS 2         /* Bt streamed once per 128 rows, k split over the waves of a workgroup */
+#define F8MI_PLAN_TILES128 3         /* 128 x 128 or 128 x 256 tiles */
+#define F8MI_PLAN_TILES256 4         /* 256 x 256 tiles, 16x16x128 MFMA, operands through LDS-DMA */
+#define F8MI_PLAN_TILES256_AND_128 5 /* the same for the tile rows of whole rounds, 128-row tiles for the rest */
+#define F8MI_PLAN_TILES256_MFMA32 6  /* 256 x 256 tiles, 32x32x64 MFMA (k % 128 == 64) */
+#define F8MI_PLAN_STAGED 7           /* 256 x 256 tiles, register-staged (ragged or short k, unaligned operands) */
+int f8mi_gemm_plan(int64_t m, int64_t n, int64_t k, int aligned, int64_t workspace_bytes);
+
 /* f8mi_gemm_nt_kb with operands that may be given transposed, so that one k-blocked copy of a tensor serves
  * both GEMMs that use it (no transposed fp8 copies at all):
  *   a, a_transposed = 0: [k/64][m][64] as above;  = 1: [m/64][k][64], i.e. the matrix [k][m] k-blocked over m

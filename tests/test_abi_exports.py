@@ -85,3 +85,31 @@ def test_cpu_tensors_are_refused_loudly():
         _native.amax_scale(torch.ones(4, 4, dtype=torch.bfloat16), torch.float8_e4m3fn)
     with pytest.raises(_native.Float8NativeError):
         _native.cast(torch.ones(4, 4, dtype=torch.bfloat16), torch.tensor(1.0), torch.float8_e4m3fn)
+
+
+def test_gemm_plan_names_the_kernel_each_shape_class_takes():
+    """f8mi_gemm_plan needs no GPU: the shape classes the GPU tests are written for really take the kernel they name."""
+    from float8_experimental_amd import _native as nat
+
+    plan = nat.gemm_plan
+    # training shapes of the benchmark: whole rounds of 256 x 256 tiles
+    for m, n, k in ((16384, 10240, 8192), (16384, 8192, 8192), (16384, 57344, 8192), (16384, 8192, 28672), (8192, 57344, 16384)):
+        assert plan(m, n, k) == ("tiles256", 0, 0), (m, n, k)
+    # decode steps stream the weight once; so does a narrow weight up to 256 rows
+    for m, n, k in ((1, 8192, 8192), (16, 57344, 8192), (32, 8192, 8192), (128, 4096, 4096), (200, 4096, 4096)):
+        assert plan(m, n, k)[0] == "few_rows", (m, n, k)
+    # a wide weight at 17 - 256 rows, and outputs of at most 256 small tiles: 128-row tiles
+    assert plan(64, 28672, 512) == ("tiles128", 0, 1) and plan(20, 16384, 256) == ("tiles128", 0, 1)
+    assert plan(200, 8192, 512) == ("tiles128", 0, 1) and plan(300, 520, 1024) == ("tiles128", 0, 1)
+    assert plan(1024, 8192, 1024) == ("tiles128", 0, 2) and plan(8192, 1024, 4096) == ("tiles128", 0, 2)
+    # few tiles and a long k: split over k when there is scratch memory, and only then
+    for m, n, k in ((256, 2048, 16384), (512, 1024, 8192), (100, 4096, 16384), (128, 8192, 28672)):
+        name, parts, mid = plan(m, n, k)
+        assert name == "tiles128_split_k" and parts in (2, 4, 8) and k % (128 * parts) == 0 and parts * m * n * 4 <= nat.GEMM_WORKSPACE_BYTES
+        assert plan(m, n, k, split_k=False)[0] in ("few_rows", "tiles128")
+    # a sparse last round goes to 128-row tiles
+    assert plan(4352, 4096, 512) == ("tiles256_and_128", 0, 1) and plan(6144, 4096, 640) == ("tiles256_and_128", 0, 2)
+    # the other contraction lengths and unaligned operands
+    assert plan(4096, 4096, 448)[0] == "tiles256_mfma32" and plan(4096, 4096, 200)[0] == "staged"
+    assert plan(4096, 4096, 4096, aligned=False)[0] == "staged" and plan(64, 4096, 4096, aligned=False)[0] == "staged"
+    assert plan(0, 4096, 4096) == (None, 0, 0)
