@@ -464,6 +464,33 @@ def test_gemm_split_over_k(nat, m, n, k):
     _gemm_check(nat, m, n, k, "e4m3", "e5m2", torch.bfloat16, seed=m + n, bias=True)
 
 
+def test_gemm_split_over_k_random_shapes(nat):
+    """Seeded shapes around the limits of the split (rows, ragged n, parts of k): whatever the plan, the result with
+    the scratch buffer agrees with the one without to fp32 accuracy, and some of the shapes do get split."""
+    import random
+
+    rng = random.Random(1234)
+    sa, sb = torch.tensor(2.0, device=DEV), torch.tensor(0.25, device=DEV)
+    split = 0
+    for case in range(14):
+        m = rng.choice([17, 33, 64, 100, 128, 129, 200, 256, 257, 384, 512, 640])
+        n = 4 * rng.randint(64, 768)
+        k = 128 * rng.choice([32, 40, 64, 96, 112, 128, 192])
+        name, parts, _ = nat.gemm_plan(m, n, k)
+        split += name == "tiles128_split_k"
+        a = _rand_fp8((m, k), torch.float8_e4m3fn, case, 4.0).to(DEV)
+        bt = _rand_fp8((n, k), torch.float8_e4m3fn, case + 100, 4.0).to(DEV)
+        with_ws = nat.gemm_nt(a, sa, bt, sb, torch.float32)
+        without = nat.gemm_nt(a, sa, bt, sb, torch.float32, split_k=False)
+        tol = 1e-5 if nat.gemm_plan(m, n, k, split_k=False)[0] != "few_rows" or name == "tiles128_split_k" else 0.0
+        err = ((with_ws - without).abs().max() / without.abs().max()).item()
+        assert err <= max(tol, 1e-5), (m, n, k, name, parts, err)
+        if name != "tiles128_split_k":
+            assert torch.equal(with_ws, without), (m, n, k, name)
+        assert torch.equal(nat.gemm_nt_kb(_to_kb(a), sa, _to_kb(bt), sb, torch.float32), with_ws), (m, n, k, name)
+    assert split >= 3, split
+
+
 # More than one round of 256 x 256 tiles with few tiles in the last one: the last tile rows go to a 128-row-tile kernel.
 @pytest.mark.parametrize("m,n,k,m_pad", [(4352, 4096, 512, 8192),      # 272 tiles: 16 of them as 128 x 128 tiles
                                          (8500, 2048, 384, 16384),     # ragged last tile row
