@@ -37,6 +37,7 @@ EXPORTS = (
     "f8mi_cast",
     "f8mi_cast_layout",
     "f8mi_cast_dynamic",
+    "f8mi_cast_dynamic_static",
     "f8mi_gemm_nt",
     "f8mi_gemm_nt_kb",
     "f8mi_gemm_kb_ex",
@@ -91,6 +92,8 @@ def lib() -> C.CDLL:
         L.f8mi_cast_layout.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, i32, vp, i32, fp, vp]
         L.f8mi_cast_dynamic.restype = i32
         L.f8mi_cast_dynamic.argtypes = [vp, i64, i64, i64, i32, i32, fp, vp, i32, vp, i32, vp, vp]
+        L.f8mi_cast_dynamic_static.restype = i32
+        L.f8mi_cast_dynamic_static.argtypes = [vp, i64, i64, i64, i32, i32, fp, vp, i32, vp, i32, vp]
         L.f8mi_gemm_nt_kb.restype = i32
         L.f8mi_gemm_nt_kb.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_kb_ex.restype = i32
@@ -378,6 +381,28 @@ def cast_dynamic(x: torch.Tensor, float8_dtype: torch.dtype, want_out: bool = Tr
                                  ws.data_ptr(), _stream(x))
     _check(rc, "f8mi_cast_dynamic")
     return out, out_t, scale
+
+
+def cast_dynamic_static(x: torch.Tensor, scale_out: torch.Tensor, out: Optional[torch.Tensor] = None,
+                        out_t: Optional[torch.Tensor] = None, out_kblock: bool = False, out_t_kblock: bool = False) -> None:
+    """``cast_dynamic`` into tensors the caller already holds, through the library's own static scratch: this
+    function and the library call behind it allocate nothing (see f8mi_cast_dynamic_static).  ``x`` must be a 2-D
+    view with unit column stride; ``out`` / ``out_t`` are fp8 tensors of rows*cols elements, ``scale_out`` one fp32
+    element.  Calls on one GPU must not overlap in time."""
+    _require_gpu(x, "x")
+    assert x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= x.shape[1], "x: 2-D with unit column stride (no copy is made here)"
+    rows, cols = x.shape
+    assert out is not None or out_t is not None, "no output requested"
+    f8 = (out if out is not None else out_t).dtype
+    for o in (out, out_t):
+        if o is not None:
+            assert o.dtype == f8 and o.dtype in _F8 and o.numel() == rows * cols and o.is_contiguous() and o.device == x.device
+    assert scale_out.dtype == torch.float32 and scale_out.numel() == 1 and scale_out.device == x.device
+    _check_device(x.device)
+    rc = lib().f8mi_cast_dynamic_static(x.data_ptr(), rows, cols, x.stride(0), _DT[x.dtype], _F8[f8], scale_out.data_ptr(),
+                                        out.data_ptr() if out is not None else None, int(out_kblock),
+                                        out_t.data_ptr() if out_t is not None else None, int(out_t_kblock), _stream(x))
+    _check(rc, "f8mi_cast_dynamic_static")
 
 
 def gemm_nt_kb(a_kb: torch.Tensor, a_scale: torch.Tensor, bt_kb: torch.Tensor, b_scale: torch.Tensor,

@@ -12,6 +12,8 @@
 // (so the 64 lanes of a store hit 32 banks twice: the floor for 256 bytes), and
 // the tile is read back as 16-byte row pieces: 8 lanes = one 128-byte segment of
 // a row of the transposed output.
+#include <atomic>
+
 #include "f8mi_common.h"
 
 namespace f8mi {
@@ -441,4 +443,47 @@ extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int6
     int rc = f8mi_amax_scale(x, rows, cols, ld, in_dtype, fp8_fmt, in_dtype, in_dtype == F8MI_FP16, nullptr, scale_dev, workspace, stream_);
     if (rc || n == 0 || (!out && !out_t)) return rc;
     return f8mi_cast_layout(x, rows, cols, ld, in_dtype, scale_dev, in_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, nullptr, stream_);
+}
+
+namespace f8mi {
+
+// ---- dynamic scaling for callers that cannot allocate ---------------------------------------------------------
+// The per-workgroup partial maxima of the amax pass (one word per workgroup, at most WS_WORDS of them whatever the
+// tensor's size) go to a device array that is part of the library's code object instead of a workspace the caller
+// brings.  Every GPU holds its own copy of the array at its own address from the moment the library is loaded on
+// it until the process ends; `scratch` below is only the host-side handle of it, the address is looked up once per
+// device and kept.  Nothing in it has to start at zero: a call writes the words it reads back.
+static __device__ __align__(256) uint32_t scratch[WS_WORDS];
+static_assert(sizeof(scratch) == F8MI_STATIC_SCRATCH_BYTES, "f8mi.h states the size of the static scratch");
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static std::atomic<uint32_t*> g_scratch_ptr[STATIC_MAX_DEVICES];
+
+// Device address of `scratch` on the current device (nullptr + error message on failure).
+static uint32_t* static_scratch_ptr() {
+    int dev = -1;
+    if (check_hip(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) { set_error("f8mi_cast_dynamic_static: device index %d, at most %d devices", dev, STATIC_MAX_DEVICES); return nullptr; }
+    uint32_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    void* addr = nullptr;
+    if (check_hip(hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+    if (!addr) { set_error("f8mi_cast_dynamic_static: the static scratch has no address on device %d", dev); return nullptr; }
+    g_scratch_ptr[dev].store((uint32_t*)addr, std::memory_order_release);  // two threads racing here store the same value
+    return (uint32_t*)addr;
+}
+
+}  // namespace f8mi
+
+extern "C" int f8mi_cast_dynamic_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt, float* scale_dev,
+                                        uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout, void* stream) {
+    if (rows < 0 || cols < 0) { set_error("f8mi_cast_dynamic_static: bad shape rows=%lld cols=%lld", (long long)rows, (long long)cols); return F8MI_ERR_INVALID_ARG; }
+    if (rows > 0 && cols > F8MI_STATIC_MAX_ELEMS / rows) {
+        set_error("f8mi_cast_dynamic_static: %lld x %lld elements, at most %lld per call (use f8mi_cast_dynamic with a workspace)",
+                  (long long)rows, (long long)cols, (long long)F8MI_STATIC_MAX_ELEMS);
+        return F8MI_ERR_INVALID_ARG;
+    }
+    uint32_t* ws = f8mi::static_scratch_ptr();
+    if (!ws) return F8MI_ERR_HIP;
+    return f8mi_cast_dynamic(x, rows, cols, ld, in_dtype, fp8_fmt, scale_dev, out, out_layout, out_t, out_t_layout, ws, stream);
 }

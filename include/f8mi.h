@@ -175,6 +175,21 @@ int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int 
 int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt, float* scale_dev,
                       uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout, void* workspace, void* stream);
 
+/* f8mi_cast_dynamic without the workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc) and so have no workspace to bring.  No
+ * counterpart in the reference.  The per-workgroup partial maxima go to an array of F8MI_STATIC_SCRATCH_BYTES that is
+ * part of the library's device code: every GPU the library runs on holds it from load until the process ends.  The
+ * call allocates and frees nothing (the first call on a device looks the array's address up, once).  Same kernels,
+ * same result bits as f8mi_cast_dynamic.  All calls on one GPU share the one array: calls that can overlap in time
+ * on the same GPU (two streams, two host threads) race on it -- give such callers f8mi_cast_dynamic and a workspace
+ * each.  The array keeps the last call's contents; nothing in it needs to start at zero.  Tensors of more than
+ * F8MI_STATIC_MAX_ELEMS elements are refused with F8MI_ERR_INVALID_ARG. */
+#define F8MI_STATIC_SCRATCH_BYTES 4096
+#define F8MI_STATIC_MAX_ELEMS (1ll << 36)
+int f8mi_cast_dynamic_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt,
+                             float* scale_dev, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
+                             void* stream);
+
 /* f8mi_gemm_nt on k-blocked operands: a = [k/64][m][64], bt = [k/64][n][64], both 16-byte
  * aligned.  Needs k % 64 == 0 and k >= 384 (F8MI_ERR_UNSUPPORTED otherwise: keep such operands
  * row-major and call f8mi_gemm_nt).  Same arithmetic, same result bits as f8mi_gemm_nt. */

@@ -72,6 +72,9 @@ def test_host_side_argument_checks_need_no_gpu():
     assert rc == -1
     rc = lib.f8mi_cast_dynamic(None, i64(4), i64(4), i64(4), 0, 0, None, None, 0, None, 0, None, None)
     assert rc == -1 and b"scale" in lib.f8mi_last_error()
+    rc = lib.f8mi_cast_dynamic_static(ctypes.c_void_p(16), i64(1 << 20), i64(1 << 20), i64(1 << 20), 0, 0, ctypes.c_void_p(16),
+                                      ctypes.c_void_p(16), 0, None, 0, None)
+    assert rc == -1 and b"at most" in lib.f8mi_last_error()
     rc = lib.f8mi_amax_scale_multi(None, 5000, i64(5000), 0, 0, 0, 0, ctypes.c_void_p(8), None, None, None)
     assert rc == -1 and b"at most" in lib.f8mi_last_error()
 
