@@ -90,6 +90,24 @@ def timed(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def probe_mfma(torch, random_data, iters=4000):
+    """TFLOP/s of a register-only fp8 MFMA loop on every CU: the matrix cores' ceiling with no memory traffic, on zero
+    operands (clock limit) or random ones (power limit).  From libf8mi_probe.so, a bench-only helper next to the library."""
+    import ctypes as C
+
+    path = os.path.join(ROOT, "float8_experimental_amd", "libf8mi_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path)
+    lib.f8mi_probe_mfma.restype = C.c_int
+    lib.f8mi_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_double), C.c_void_p]
+    scratch = torch.empty(1 << 20, dtype=torch.uint8, device="cuda:0")
+    out = C.c_double(0.0)
+    rc = lib.f8mi_probe_mfma(int(random_data), iters, scratch.data_ptr(), scratch.numel(), C.byref(out),
+                             torch.cuda.current_stream().cuda_stream)
+    return out.value if rc == 0 else None
+
+
 def cpu_baseline(torch, target_s):
     """The oracle's emulate=True restatement (fp32 dequant + torch.mm on the host) on token slices of the benchmark
     shapes, smallest weight first, until about ``target_s`` seconds of CPU work have been timed."""
@@ -204,8 +222,8 @@ def main():
         bf16_step = sum(v["bf16_ms"] for v in per_shape.values()) * 1e-3
 
     # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
-    mfma_zero = _native.probe_mfma(False)
-    mfma_random = _native.probe_mfma(True)
+    mfma_zero = probe_mfma(torch, False)
+    mfma_random = probe_mfma(torch, True)
 
     out = {
         "metric": "Float8Linear fwd+bwd TFLOP/s at LLaMa-2-70B shapes (1 GPU); cast GB/s",
@@ -240,7 +258,7 @@ def main():
             "flop_per_launch": flop_gemm / max(n_gemm, 1),
             "mfma_only_zero_operands_TFLOP/s": mfma_zero,
             "mfma_only_random_operands_TFLOP/s": mfma_random,
-            "frac_of_mfma_only_random": gemm_tflops / mfma_random if mfma_random > 0 else None,
+            "frac_of_mfma_only_random": gemm_tflops / mfma_random if mfma_random else None,
         },
         "hbm_kernels": hbm,
         "per_shape": per_shape,

@@ -8,6 +8,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libf8mi.so")
+# bench-only helper (register-only MFMA loop), kept out of libf8mi.so: it synchronises and copies from the host
+PROBE_SRC = os.path.join(CSRC, "bench", "f8mi_probe.hip")
+PROBE_LIB = os.path.join(HERE, "libf8mi_probe.so")
 OBJ_DIR = os.path.join(CSRC, "build")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -40,6 +43,7 @@ def build(verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         objs = list(ex.map(_compile, srcs))
     subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], check=True)
+    subprocess.run([HIPCC, *FLAGS, "-shared", PROBE_SRC, "-o", PROBE_LIB], check=True)
     if verbose:
         print(f"built {LIB} from {len(srcs)} sources", file=sys.stderr)
     return LIB

@@ -46,7 +46,6 @@ EXPORTS = (
     "f8mi_prof_enable",
     "f8mi_prof_reset",
     "f8mi_prof_read",
-    "f8mi_probe_mfma",
 )
 
 _lib = None
@@ -116,8 +115,6 @@ def lib() -> C.CDLL:
         L.f8mi_prof_reset.argtypes = []
         L.f8mi_prof_read.restype = i32
         L.f8mi_prof_read.argtypes = [i32, C.POINTER(C.c_uint64), C.POINTER(C.c_double), C.POINTER(C.c_double)]
-        L.f8mi_probe_mfma.restype = i32
-        L.f8mi_probe_mfma.argtypes = [i32, i32, vp, C.c_size_t, C.POINTER(C.c_double), vp]
         _lib = L
     return _lib
 
@@ -563,17 +560,3 @@ def prof_read(kernel: int):
     n, ms, work = C.c_uint64(0), C.c_double(0), C.c_double(0)
     _check(lib().f8mi_prof_read(kernel, C.byref(n), C.byref(ms), C.byref(work)), "f8mi_prof_read")
     return n.value, ms.value, work.value
-
-
-def probe_mfma(random_data: bool, iters: int = 4000, device: Optional[torch.device] = None) -> float:
-    """TFLOP/s of a register-only fp8 MFMA loop on every CU (see f8mi_probe_mfma): the matrix cores'
-    ceiling with no memory traffic, on zero operands (clock limit) or random ones (power limit)."""
-    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else device
-    _check_device(dev)
-    scratch = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
-    out = C.c_double(0.0)
-    with torch.cuda.device(dev):
-        rc = lib().f8mi_probe_mfma(int(random_data), iters, scratch.data_ptr(), scratch.numel(), C.byref(out),
-                                   _raw_stream(dev))
-    _check(rc, "f8mi_probe_mfma")
-    return out.value

@@ -1,10 +1,18 @@
-// Measurement aid: what the fp8 matrix cores of this GPU sustain with no memory traffic at all.
+// Benchmark aid, built into its own shared object (libf8mi_probe.so): what the fp8 matrix cores of this GPU
+// sustain with no memory traffic at all.  It is not part of libf8mi.so: it copies from host memory and waits for
+// the stream, which the library's entry points never do.
 // A register-only loop of v_mfma_f32_16x16x128_f8f6f4 (the GEMM's instruction) over 64 accumulator
 // tiles per wave, one wave per SIMD on every CU.  On all-zero operands the loop runs at the clock limit;
 // on random fp8 bytes it runs into the power limit, which is the ceiling a real GEMM works under.
+//
+//   int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, size_t scratch_bytes, double* tflops, void* stream)
+//     random_data 0: all-zero operands, 1: random finite e4m3 bytes;  scratch_dev: >= 1 MiB of device memory of the
+//     caller's;  *tflops receives the rate.  Returns 0, or -1 (bad argument) / -3 (a HIP call failed).
 #include <vector>
 
-#include "f8mi_common.h"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
 
 namespace f8mi {
 
@@ -48,11 +56,18 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const int* __restrict__
 
 using namespace f8mi;
 
+static int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return 0;
+    fprintf(stderr, "f8mi_probe_mfma: %s: %s\n", what, hipGetErrorString(e));
+    return -3;
+}
+
 extern "C" int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, size_t scratch_bytes, double* tflops, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
-    const int n_cu = cu_count();
+    int dev = 0, n_cu = 0;
+    if (check_hip(hipGetDevice(&dev), "hipGetDevice") || check_hip(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute")) return -3;
     const size_t need = 65536 * sizeof(int) + (size_t)n_cu * 256 * sizeof(float);
-    if (!scratch_dev || scratch_bytes < need || !tflops || iters < 1) { set_error("f8mi_probe_mfma: needs %zu bytes of device scratch, a result pointer and iters >= 1", need); return F8MI_ERR_INVALID_ARG; }
+    if (!scratch_dev || scratch_bytes < need || !tflops || iters < 1) { fprintf(stderr, "f8mi_probe_mfma: needs %zu bytes of device scratch, a result pointer and iters >= 1\n", need); return -1; }
     int* in = (int*)scratch_dev;
     float* out = (float*)((char*)scratch_dev + 65536 * sizeof(int));
     std::vector<int> h(65536, 0);
@@ -88,5 +103,5 @@ extern "C" int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, si
     if (rc) return rc;
     const double flop = 64.0 * 2 * 16 * 16 * 128 * (double)iters * 4 * n_cu;
     *tflops = flop / (ms * 1e-3) / 1e12;
-    return F8MI_OK;
+    return 0;
 }

@@ -3,6 +3,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -34,14 +35,14 @@ struct ProfRec {
 };
 
 static std::mutex g_prof_mu;
-static bool g_prof_on = false;
+static std::atomic<bool> g_prof_on{false};  // read by every launch, on any thread, without the lock
 static std::vector<ProfRec*> g_prof_recs;
 static uint64_t g_prof_launches[F8MI_K_COUNT];
 static double g_prof_ms[F8MI_K_COUNT];
 static double g_prof_work[F8MI_K_COUNT];
 
 ProfScope::ProfScope(int kernel_, double work_, hipStream_t stream_) : kernel(kernel_), work(work_), stream(stream_), rec(nullptr) {
-    if (!g_prof_on) return;
+    if (!g_prof_on.load(std::memory_order_relaxed)) return;
     ProfRec* r = new ProfRec{kernel, work, nullptr, nullptr};
     if (hipEventCreate(&r->start) != hipSuccess || hipEventCreate(&r->stop) != hipSuccess) { delete r; return; }
     (void)hipEventRecord(r->start, stream);
@@ -100,7 +101,7 @@ extern "C" int f8mi_device_info(int device, int* cu_count, int* lds_bytes, char*
 
 extern "C" int f8mi_prof_enable(int on) {
     std::lock_guard<std::mutex> lk(g_prof_mu);
-    g_prof_on = on != 0;
+    g_prof_on.store(on != 0, std::memory_order_relaxed);
     return F8MI_OK;
 }
 

@@ -277,17 +277,6 @@ static int launch_gemm1(bool aligned, int c_dtype, dim3 g, hipStream_t stream, c
 
 using namespace f8mi;
 
-// 0: default choice, 1: register-staged kernel only, 2: no 16x16x128 kernel
-static int gemm_impl() {
-    static const int v = [] {
-        const char* e = getenv("F8MI_GEMM_IMPL");
-        if (e && !strcmp(e, "staged")) return 1;
-        if (e && !strcmp(e, "dma32")) return 2;
-        return 0;
-    }();
-    return v;
-}
-
 // An output whose last round of 256 x 256 tiles would leave most CUs idle (at most 128 tiles in it) is split by
 // rows: the tile rows that fill whole rounds go to the large-tile kernel, the rest to a 128-row-tile kernel that
 // spreads them over all CUs (same accumulation order, so no output bit depends on the split).  Returns the number
@@ -316,12 +305,10 @@ static RowSplit split_last_round(int64_t tiles_m, int64_t tiles_n, int64_t k) {
 //                                                        sparse last round: 128-row tiles, see split_last_round)
 //   aligned, K % 64 == 0, K >= 384                    -> 256 x 256 tiles, 32x32x64 MFMA, LDS-DMA
 //   anything else (ragged K, unaligned, short K)      -> 256 x 256 tiles, register-staged
-// F8MI_GEMM_IMPL=staged forces the register-staged kernel, =dma32 the 32x32x64 LDS-DMA kernel (comparison runs).
 struct GemmPlan { int kind; int parts; int mid; RowSplit split; };
 static GemmPlan gemm_plan(int64_t m, int64_t n, int64_t k, bool aligned, int64_t ws_bytes) {
     GemmPlan p{F8MI_PLAN_STAGED, 0, 0, {0, 0}};
-    const int impl = gemm_impl();
-    if (aligned && impl == 0) {
+    if (aligned) {
         if (const int parts = pick_k_splits(m, n, k, ws_bytes)) {
             p.kind = F8MI_PLAN_TILES128_SPLIT_K; p.parts = parts; p.mid = use_mid_tiles(m, n, k);
             return p;
@@ -329,10 +316,10 @@ static GemmPlan gemm_plan(int64_t m, int64_t n, int64_t k, bool aligned, int64_t
         if (use_skinny(m, n, k)) { p.kind = F8MI_PLAN_FEW_ROWS; return p; }
         if (const int mid = use_mid_tiles(m, n, k)) { p.kind = F8MI_PLAN_TILES128; p.mid = mid; return p; }
     }
-    if (aligned && k >= 384 && k % 64 == 0 && impl != 1) {
-        if (k % 128 == 0 && impl != 2) {
+    if (aligned && k >= 384 && k % 64 == 0) {
+        if (k % 128 == 0) {
             const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
-            p.split = impl == 0 ? split_last_round(tiles_m, tiles_n, k) : RowSplit{0, 0};
+            p.split = split_last_round(tiles_m, tiles_n, k);
             p.kind = p.split.rows_large ? F8MI_PLAN_TILES256_AND_128 : F8MI_PLAN_TILES256;
             p.mid = p.split.mid;
             return p;
@@ -454,8 +441,8 @@ extern "C" int f8mi_gemm_nt_kb_ws(const void* a, int a_fmt, const void* bt, int 
         }
         default: break;
     }
-    // whole output on 256 x 256 tiles (there is no register-staged kernel for k-blocked operands: F8MI_GEMM_IMPL=staged means these)
-    if (k % 128 == 0 && gemm_impl() != 2)
+    // whole output on 256 x 256 tiles (there is no register-staged kernel for k-blocked operands)
+    if (k % 128 == 0)
         return launch_gemm_dma16(a_fmt, b_fmt, c_dtype, g, stream, A, 64, a_unit, B, 64, b_unit, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev,
                                  (int)tiles_m, (int)tiles_n, c_vec_ok);
     return launch_gemm_dma(a_fmt, b_fmt, c_dtype, g, stream, A, 64, a_unit, B, 64, b_unit, M, N, K, scale_a_dev, scale_b_dev, c, ldc, bias_dev,

@@ -282,15 +282,6 @@ int f8mi_prof_enable(int on);
 int f8mi_prof_reset(void);
 int f8mi_prof_read(int kernel, uint64_t* launches, double* total_ms, double* total_work);
 
-/*
- * Measurement aid (no counterpart in the reference): the rate the fp8 matrix cores sustain with no
- * memory traffic, in TFLOP/s -- a register-only loop of the GEMM's MFMA instruction on every CU, on
- * all-zero operands (random_data = 0: the clock limit) or on random fp8 bytes (random_data = 1: the
- * power limit a real GEMM runs under).  Synchronises the stream.  `scratch_dev`: at least 1 MiB of
- * device memory the caller owns.
- */
-int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, size_t scratch_bytes, double* tflops, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -34,6 +34,15 @@ def test_library_exports_every_declared_symbol():
     assert 8 <= lib.f8mi_workspace_bytes() <= 4096
 
 
+def test_benchmark_probe_is_not_part_of_the_library():
+    """The register-only MFMA probe synchronises and copies from the host: it lives in its own shared object."""
+    lib = ctypes.CDLL(LIB)
+    assert not hasattr(lib, "f8mi_probe_mfma")
+    probe = os.path.join(ROOT, "float8_experimental_amd", "libf8mi_probe.so")
+    assert os.path.exists(probe), f"{probe} has not been built (run __graft_entry__.build())"
+    assert hasattr(ctypes.CDLL(probe), "f8mi_probe_mfma")
+
+
 def test_binding_lists_the_same_symbols():
     from float8_experimental_amd import _native
 

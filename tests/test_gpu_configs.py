@@ -1,5 +1,7 @@
-"""The benchmark configurations that are not the bench line, at their full sizes, as parity cases.
+"""The benchmark configurations at their full sizes, as parity cases.
 
+config 2: the bench line's own workload -- the four LLaMa-2-70B shapes at 16384 tokens, dynamic scaling, one fwd+bwd
+          through Float8Linear's one-fp8-copy-per-tensor route (cast_dynamic -> gemm_nt_kb / gemm_kb_ex).
 config 3: the four LLaMa-2-70B shapes with delayed scaling everywhere, history 16, 20 iterations with the
           activations growing x1.1 per step and a sync before every forward.
 config 4: a Llama-3-8B-shaped 4-layer decoder (d=4096, ffn=14336, 32 heads / 8 KV heads, seq 8192, batch 1,
@@ -71,9 +73,69 @@ def _sampled_linear_check(to, x, w, dy, y, dx, dw, sx, sw, sg, seed, what):
     return x8, g8
 
 
-# ------------------------------------------------------------------ config 3
-
 SHAPES = [("wqkv", 8192, 10240), ("wo", 8192, 8192), ("w13", 8192, 57344), ("w2", 28672, 8192)]
+
+
+# ------------------------------------------------------------------ config 2
+
+def _kb_rows(t_kb, rows):
+    """Rows `rows` of a k-blocked fp8 tensor [cols/64, R, 64] as row-major bytes [len(rows), cols] on the CPU."""
+    return t_kb.view(torch.uint8)[:, rows, :].permute(1, 0, 2).reshape(len(rows), -1).cpu()
+
+
+@pytest.mark.parametrize("name,k,n", SHAPES)
+def test_config2_dynamic_scaling_at_llama70b_shapes(f8, name, k, n):
+    """Float8Linear.from_float with the default (all dynamic) config, x ~ N(0,1), kaiming-uniform W, dY ~ N(0, 1e-2),
+    fwd + bwd at 16384 tokens: the three scales bit-exact against the oracle's tensor_to_scale of the same tensors
+    (reference float8_utils.py:102-120), the fp8 bytes the module multiplied -- sampled rows of its saved x8 / W8 and
+    of dY8 -- bit-exact against the oracle's cast (float8_tensor.py:158-159, float8_utils.py:123-139), and y / dx / dw
+    on sampled rows and columns within 1e-2 (of the output's scale) of the emulated matmul (float8_aten_api.py:16-28)."""
+    from float8_experimental_amd import _native
+
+    to = _oracle()
+    m = 16384
+    assert _native.tn_ok(m, k, n), "config 2 must run the one-copy route (gemm_nt_kb forward, gemm_kb_ex backward)"
+    torch.manual_seed({"wqkv": 20, "wo": 21, "w13": 22, "w2": 23}[name])
+    lin = nn.Linear(k, n, bias=False, device=DEV, dtype=torch.bfloat16)  # default init: kaiming-uniform
+    mod = f8.Float8Linear.from_float(lin)
+    assert mod.scaling_repr() == "i:dyn,w:dyn,go:dyn"
+    x = torch.randn(m, k, device=DEV, dtype=torch.bfloat16).requires_grad_()
+    dy = (torch.randn(m, n, device=DEV, dtype=torch.float32) * 1e-2).to(torch.bfloat16)
+    y = mod(x)
+    fn = y.grad_fn
+    assert type(fn).__name__ == "_float8_linear_fnBackward" and fn.kb is None  # kb None: one k-blocked copy per tensor
+    x8_kb, w8_kb, sx_dev, sw_dev = fn.saved_tensors
+    assert tuple(x8_kb.shape) == (k // 64, m, 64) and tuple(w8_kb.shape) == (k // 64, n, 64)
+    y.backward(dy)
+    w = mod.weight.detach()
+
+    # scales: bit-exact (the CPU reduction over the whole tensor is the oracle's own)
+    sx, sw, sg = to.tensor_to_scale(x.detach().cpu(), E4M3), to.tensor_to_scale(w.cpu(), E4M3), to.tensor_to_scale(dy.cpu(), E5M2)
+    assert sx_dev.cpu().item() == sx.item(), (name, "input scale", sx_dev.item(), sx.item())
+    assert sw_dev.cpu().item() == sw.item(), (name, "weight scale", sw_dev.item(), sw.item())
+    # dY's copy lives only inside backward: the same library call the module makes there
+    g8_kb, _, sg_dev = _native.cast_dynamic(dy, E5M2, want_out=True, out_kblock=True)
+    assert sg_dev.cpu().item() == sg.item(), (name, "grad_output scale", sg_dev.item(), sg.item())
+
+    # fp8 bytes of sampled rows: bit-exact
+    g = torch.Generator().manual_seed(1)
+    rm = torch.randperm(m, generator=g)[:32]
+    rn = torch.randperm(n, generator=g)[:32]
+    rows_first_last = lambda r, total: torch.cat([r, torch.tensor([0, total - 1])])
+    rm, rn = rows_first_last(rm, m), rows_first_last(rn, n)
+    want = to.cast_to_fp8(x.detach()[rm.to(DEV)].cpu(), sx, E4M3).view(torch.uint8)
+    assert torch.equal(_kb_rows(x8_kb, rm.to(DEV)), want), (name, "x8 bytes")
+    want = to.cast_to_fp8(w[rn.to(DEV)].cpu(), sw, E4M3).view(torch.uint8)
+    assert torch.equal(_kb_rows(w8_kb, rn.to(DEV)), want), (name, "w8 bytes")
+    want = to.cast_to_fp8(dy[rm.to(DEV)].cpu(), sg, E5M2).view(torch.uint8)
+    assert torch.equal(_kb_rows(g8_kb, rm.to(DEV)), want), (name, "dy8 bytes")
+    del g8_kb
+
+    # the three products on sampled rows / columns, within 1e-2 of the emulated reference
+    _sampled_linear_check(to, x.detach(), w, dy, y.detach(), x.grad, mod.weight.grad, sx, sw, sg, 200 + len(name), f"config2 {name}")
+
+
+# ------------------------------------------------------------------ config 3
 
 
 def test_config3_delayed_scaling_20_iterations_at_llama70b_shapes(f8):

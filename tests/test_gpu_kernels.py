@@ -812,12 +812,3 @@ def test_tensors_of_more_than_2_31_elements(nat):
         assert torch.equal(c[r0:r0 + 256], ref), r0
     exact = a8[rows - 64:].double() @ b8.double().t()
     torch.testing.assert_close(c[rows - 64:].double(), exact, rtol=2.0**-7, atol=0.5)
-
-
-def test_mfma_probe_reports_a_sane_ceiling(nat):
-    """f8mi_probe_mfma: register-only MFMA loop; zeros run at the clock limit, random bytes below it."""
-    zero = nat.probe_mfma(False, iters=1000)
-    rnd = nat.probe_mfma(True, iters=1000)
-    assert 2000.0 < rnd <= zero * 1.02 and zero < 5300.0, (zero, rnd)
-    L = nat.lib()
-    assert L.f8mi_probe_mfma(0, 10, None, 0, None, None) != 0  # no scratch: refused on the host
