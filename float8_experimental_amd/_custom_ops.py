@@ -1,5 +1,9 @@
-"""The fused linear as two ``torch.library`` custom ops, so that ``torch.compile`` sees one opaque node per
-direction instead of tracing into the ctypes calls (which it cannot).
+"""The kernels as ``torch.library`` custom ops, so that ``torch.compile`` sees opaque nodes with known shapes
+instead of tracing into the ctypes calls (which it cannot): the fused linear as one node per direction, and the
+primitives the Float8Tensor-level API is made of -- amax + scale, the saturated cast, the scaled matmul -- as one
+node each (``f8mi::amax_scale``, ``f8mi::cast``, ``f8mi::gemm_nt``), which is what lets code that produces or
+consumes a ``Float8Tensor`` compile (graph inputs, graph outputs, breaks in the middle; reference
+test/test_compile.py:173-254).
 
 The reference keeps its float8 pieces traceable with ``torch._dynamo.allow_in_graph``
 (float8_linear.py:43, float8_tensor.py:131,198) and lets inductor generate the casts; here the kernels
@@ -18,9 +22,57 @@ from typing import List, Optional, Tuple
 import torch
 
 from . import _native
-from .float8_utils import e4m3_dtype, e5m2_dtype
 
+e4m3_dtype, e5m2_dtype = torch.float8_e4m3fn, torch.float8_e5m2  # as float8_utils (which imports this module)
 _KB = _native.KB
+
+
+# ---- the primitives ------------------------------------------------------------------------------------------
+
+@torch.library.custom_op("f8mi::amax_scale", mutates_args=())
+def amax_scale(x: torch.Tensor, float8_dtype: torch.dtype, math_dtype: torch.dtype, orig_is_fp16: bool) -> Tuple[
+        torch.Tensor, torch.Tensor]:
+    """(max|x|, fp8 scale of it), both 0-dim fp32, in one pass over x: ``tensor_to_amax`` + ``amax_to_scale`` of the
+    reference (float8_utils.py:35-57, 102-120) with the scale arithmetic rounded to ``math_dtype``."""
+    return _native.amax_scale(x, float8_dtype, math_dtype=math_dtype, orig_is_fp16=orig_is_fp16)
+
+
+@amax_scale.register_fake
+def _(x, float8_dtype, math_dtype, orig_is_fp16):
+    return (torch.empty((), dtype=torch.float32, device=x.device), torch.empty((), dtype=torch.float32, device=x.device))
+
+
+@torch.library.custom_op("f8mi::cast", mutates_args=())
+def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, product_dtype: torch.dtype,
+         want_amax: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(fp8 bytes of clamp(x * scale) with x's shape, max|x| as [1] fp32 or an empty tensor): the saturated cast of
+    the reference (float8_tensor.py:158-159, float8_utils.py:123-139), optionally with the amax pass of delayed
+    scaling (float8_scaling_utils.py:89) folded in.  ``product_dtype``: what ``x * scale`` is rounded to."""
+    amax = torch.empty(1 if want_amax else 0, dtype=torch.float32, device=x.device)
+    bits, _ = _native.cast(x, scale, float8_dtype, product_dtype=product_dtype, amax_out=amax if want_amax else None)
+    return bits, amax
+
+
+@cast.register_fake
+def _(x, scale, float8_dtype, product_dtype, want_amax):
+    return (torch.empty(x.shape, dtype=float8_dtype, device=x.device),
+            torch.empty(1 if want_amax else 0, dtype=torch.float32, device=x.device))
+
+
+@torch.library.custom_op("f8mi::gemm_nt", mutates_args=())
+def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: torch.Tensor, out_dtype: torch.dtype,
+            bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``(a @ bt^T) / (a_scale * b_scale) (+ bias)`` on the matrix cores: ``torch._scaled_mm`` as the reference calls it
+    (float8_python_api.py:24-64), with the second operand given as [n, k]."""
+    return _native.gemm_nt(a, a_scale, bt, b_scale, out_dtype, bias=bias)
+
+
+@gemm_nt.register_fake
+def _(a, a_scale, bt, b_scale, out_dtype, bias):
+    return torch.empty((a.shape[0], bt.shape[0]), dtype=out_dtype, device=a.device)
+
+
+# ---- the fused linear ----------------------------------------------------------------------------------------
 
 
 def _layout(t_rows: int, t_cols: int, kblock: bool):
@@ -141,7 +193,7 @@ class _LinearFn(torch.autograd.Function):
         xs, ws, sx, sw = ctx.saved_tensors
         need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         bufs_g = ctx.bufs_g
-        dx, dw, ag = linear_bwd(gy.contiguous(), xs, ws, sx, sw, ctx.k, need_dx, need_dw,
+        dx, dw, ag = linear_bwd(gy, xs, ws, sx, sw, ctx.k, need_dx, need_dw,
                                 bufs_g[1] if bufs_g is not None else None)
         if bufs_g is not None:
             bufs_g[0].copy_(ag)

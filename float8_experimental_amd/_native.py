@@ -206,9 +206,15 @@ def gemm_plan(m: int, n: int, k: int, aligned: bool = True, split_k: bool = True
 
 
 def _as_2d(x: torch.Tensor) -> Tuple[torch.Tensor, int, int, int]:
-    """(tensor whose memory is read, rows, cols, row stride) -- copies only when the layout needs it."""
+    """(tensor whose memory is read, rows, cols, row stride) -- copies only when the layout needs it.  A tensor
+    expanded over all its leading dimensions (what autograd hands to backward after ``y.sum()``) is passed as ONE row
+    with row stride 0: the kernels read that row for every output row, nothing of rows x cols is materialised."""
     if x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= x.shape[1] and x.shape[0] > 0 and x.shape[1] > 0:
         return x, x.shape[0], x.shape[1], x.stride(0)
+    if x.dim() >= 2 and x.shape[-1] > 0 and x.numel() > x.shape[-1] and all(
+            st == 0 or sz == 1 for st, sz in zip(x.stride()[:-1], x.shape[:-1])):
+        row = x[(0,) * (x.dim() - 1)].contiguous()
+        return row, x.numel() // x.shape[-1], x.shape[-1], 0
     if not x.is_contiguous():
         x = x.contiguous()
     cols = x.shape[-1] if x.dim() > 0 else 1

@@ -233,9 +233,10 @@ extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_
                                int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
                                void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
-    if (rows < 0 || cols < 0 || ld < cols) { set_error("f8mi_amax_scale: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
+    if (rows < 0 || cols < 0 || (ld < cols && ld != 0)) { set_error("f8mi_amax_scale: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
     if (in_dtype < 0 || in_dtype > 2 || math_dtype < 0 || math_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_amax_scale: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
     if (!amax_dev && !scale_dev) { set_error("f8mi_amax_scale: no output requested"); return F8MI_ERR_INVALID_ARG; }
+    if (ld == 0 && rows > 1) rows = 1;  // every row is the same `cols` elements: the maximum of one of them
     const int64_t n = rows * cols;
     if (n == 0) {
         hipLaunchKernelGGL(amax_empty_kernel, dim3(1), dim3(64), 0, stream, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);

@@ -376,7 +376,8 @@ extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64
     if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
     if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
     const int out_kb = out_layout == F8MI_LAYOUT_KBLOCK64, out_t_kb = out_t_layout == F8MI_LAYOUT_KBLOCK64;
-    if (rows < 0 || cols < 0 || ld < cols) { set_error("f8mi_cast: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
+    // ld == 0: every row reads the same `cols` elements (the kernels address row * ld + col)
+    if (rows < 0 || cols < 0 || (ld < cols && ld != 0)) { set_error("f8mi_cast: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
     if (in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
     if (product_dtype != in_dtype && product_dtype != F8MI_FP32) { set_error("f8mi_cast: product_dtype must be the input dtype or fp32"); return F8MI_ERR_INVALID_ARG; }
     if (!scale_dev) { set_error("f8mi_cast: null scale"); return F8MI_ERR_INVALID_ARG; }
@@ -401,7 +402,7 @@ extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64
         if (rc) return rc;
     }
     const double n = (double)rows * (double)cols;
-    ProfScope prof(F8MI_K_CAST, n * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
+    ProfScope prof(F8MI_K_CAST, (ld == 0 ? (double)cols : n) * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
     if (in_dtype == F8MI_BF16) {
         if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
         return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
@@ -425,7 +426,7 @@ extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int6
                                  uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout, void* workspace, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (!scale_dev) { set_error("f8mi_cast_dynamic: null scale"); return F8MI_ERR_INVALID_ARG; }
-    if (rows < 0 || cols < 0 || ld < cols || in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast_dynamic: bad shape or dtype/format code"); return F8MI_ERR_INVALID_ARG; }
+    if (rows < 0 || cols < 0 || (ld < cols && ld != 0) || in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast_dynamic: bad shape or dtype/format code"); return F8MI_ERR_INVALID_ARG; }
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
     const int64_t n = rows * cols;
     if (n > 0 && rows * ((cols + 7) / 8) <= SMALL_MAX_ITEMS && (out || out_t)) {

@@ -17,7 +17,7 @@ import torch
 
 from . import _native
 from .config import Float8LinearConfig, ScalingType
-from .float8_aten_api import mm_float8_emulated
+from . import float8_aten_api  # noqa: F401  (registers torch.ops.aten.mm_float8_emulated)
 from .float8_scaling_utils import (
     _maybe_initialize_amaxes_scales_for_float8_cast,
     hp_tensor_to_float8_delayed,
@@ -37,6 +37,7 @@ from .float8_utils import e4m3_dtype, e5m2_dtype
 _KINDS = ("input", "weight", "grad_output")
 
 
+@torch._dynamo.allow_in_graph
 class manual_float8_matmul(torch.autograd.Function):
     """``input_fp8 @ weight_fp8_t`` on Float8Tensors with both backward products
     (reference float8_linear.py:43-95)."""
@@ -136,7 +137,7 @@ class _float8_linear_fn(torch.autograd.Function):
             w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx, kb_fwd, kb_dx,
                                           known_scale=mod._precomputed_weight_scale)
             if emulate:
-                y = mm_float8_emulated(x8, sx, w8.t(), sw, x.dtype)
+                y = torch.ops.aten.mm_float8_emulated(x8, sx, w8.t(), sw, x.dtype)
             else:
                 y = _gemm(x8, sx, w8, sw, x.dtype, kb_fwd)
             ctx.kb = (kb_dx, kb_dw)
@@ -167,13 +168,13 @@ class _float8_linear_fn(torch.autograd.Function):
         emulate = mod.linear_mm_config.grad_input.emulate
         if need_dx:  # grad_input = dY @ W          [M,N] x [N,K]
             if emulate:
-                dx = mm_float8_emulated(g8, sg, w8t.t(), sw, dy.dtype)
+                dx = torch.ops.aten.mm_float8_emulated(g8, sg, w8t.t(), sw, dy.dtype)
             else:
                 dx = _gemm(g8, sg, w8t, sw, dy.dtype, kb_dx)
             dx = dx.reshape(ctx.x_shape)
         if need_dw:  # grad_weight = dY^T @ x       [N,M] x [M,K]
             if emulate:
-                dw = mm_float8_emulated(g8t, sg, x8t.t(), sx, dy.dtype)
+                dw = torch.ops.aten.mm_float8_emulated(g8t, sg, x8t.t(), sx, dy.dtype)
             else:
                 dw = _gemm(g8t, sg, x8t, sx, dy.dtype, kb_dw)
         return dx, dw, None, None

@@ -66,8 +66,14 @@ def convert_to_float8_training(module: nn.Module, *, module_filter_fn: Optional[
 
 
 def get_float8_layers(model: torch.nn.Module) -> List[Float8Linear]:
-    """All Float8Linear modules of ``model`` (reference :157-169)."""
-    return [m for m in model.modules() if isinstance(m, Float8Linear)]
+    """All Float8Linear modules of ``model``; outside a compiled region their buffers are marked as living at
+    fixed addresses, so that a compiled sync or step treats them as static inputs (reference :157-169)."""
+    fp8_layers = [m for m in model.modules() if isinstance(m, Float8Linear)]
+    if not torch.compiler.is_compiling():
+        for layer in fp8_layers:
+            for buf in layer.buffers():
+                torch._dynamo.mark_static_address(buf, guard=True)
+    return fp8_layers
 
 
 def _sync_table(fp8_layers) -> torch.Tensor:

@@ -10,7 +10,7 @@ from typing import Any, Dict
 import torch
 from torch.utils._pytree import tree_map
 
-from .float8_aten_api import mm_float8_emulated
+from . import float8_aten_api  # noqa: F401  (registers torch.ops.aten.mm_float8_emulated)
 from .float8_python_api import addmm_float8_unwrapped
 from .float8_tensor import choose_scaled_mm_config, Float8Tensor
 from .float8_utils import is_row_major, pad_tensor_for_matmul
@@ -106,7 +106,7 @@ def _mm_impl(a: Float8Tensor, b: Float8Tensor, bias):
     cfg = choose_scaled_mm_config(a._gemm_input_role, a._linear_mm_config, b._gemm_input_role, b._linear_mm_config)
     output_dtype = a._orig_dtype
     if cfg.emulate:
-        out = mm_float8_emulated(a._data, a._scale, b._data, b._scale, output_dtype)
+        out = torch.ops.aten.mm_float8_emulated(a._data, a._scale, b._data, b._scale, output_dtype)
         return out if bias is None else out + bias
     return addmm_float8_unwrapped(a_data, a_scale, b_data, b_scale, output_dtype, output_scale=None, bias=bias,
                                   use_fast_accum=cfg.use_fast_accum)

@@ -5,6 +5,7 @@ from typing import Optional
 
 import torch
 
+from . import _custom_ops  # noqa: F401  (registers torch.ops.f8mi.*)
 from . import _native
 
 
@@ -24,4 +25,5 @@ def addmm_float8_unwrapped(a_data: torch.Tensor, a_scale: torch.Tensor, b_data: 
     if output_scale is not None:
         raise NotImplementedError("fp8 output of the scaled matmul is not supported")
     assert a_data.dim() == 2 and b_data.dim() == 2 and a_data.shape[1] == b_data.shape[0]
-    return _native.gemm_nt(a_data, a_scale, b_data.t(), b_scale, output_dtype, bias=bias)
+    _native._require_gpu(a_data, "a_data")
+    return torch.ops.f8mi.gemm_nt(a_data, a_scale, b_data.t(), b_scale, output_dtype, bias)

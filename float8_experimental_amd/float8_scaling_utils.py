@@ -50,6 +50,7 @@ def _maybe_initialize_amaxes_scales_for_float8_cast(x, cur_amax, amax_history, s
         _native.delayed_init(cur_amax, amax_history, scale, float8_dtype, x.dtype == torch.float16)
 
 
+@torch._dynamo.allow_in_graph
 class NoopFwToFloat8E5M2BwDelayed(torch.autograd.Function):
     """Identity in forward; casts the gradient to e5m2 with delayed scaling in backward
     (reference float8_scaling_utils.py:128-185)."""
@@ -73,6 +74,7 @@ class NoopFwToFloat8E5M2BwDelayed(torch.autograd.Function):
         return res, None, None, None, None, None, None
 
 
+@torch._dynamo.allow_in_graph
 class NoopFwToFloat8E5M2BwDynamic(torch.autograd.Function):
     """Identity in forward; casts the gradient to e5m2 with dynamic scaling in backward
     (reference float8_scaling_utils.py:188-216)."""

@@ -69,15 +69,19 @@ def _product_dtype(hp: torch.Tensor, scale: torch.Tensor) -> torch.dtype:
     return torch.promote_types(hp.dtype, scale.dtype)
 
 
+@torch._dynamo.allow_in_graph
 class _ToFloat8ConstrFunc(torch.autograd.Function):
-    """High precision -> Float8Tensor; the gradient passes through unchanged (reference :131-195)."""
+    """High precision -> Float8Tensor; the gradient passes through unchanged (reference :131-195).
+    The cast is the custom op ``f8mi::cast``: one opaque node when ``torch.compile`` traces this function."""
 
     @staticmethod
     def forward(ctx, tensor, scale, float8_dtype=e4m3_dtype, linear_mm_config=None,
                 gemm_input_role=GemmInputRole.INPUT, amax_buffer=None):
-        # amax_buffer (delayed scaling): max|tensor| is written there by the same kernel
-        bits, _ = _native.cast(tensor, scale, float8_dtype, product_dtype=_product_dtype(tensor, scale),
-                               amax_out=amax_buffer)
+        _native._require_gpu(tensor, "tensor")
+        # amax_buffer (delayed scaling): max|tensor| comes out of the same kernel and is copied there
+        bits, amax = torch.ops.f8mi.cast(tensor, scale, float8_dtype, _product_dtype(tensor, scale), amax_buffer is not None)
+        if amax_buffer is not None:
+            amax_buffer.copy_(amax.reshape(amax_buffer.shape))
         return Float8Tensor(bits, scale, tensor.dtype, linear_mm_config=linear_mm_config,
                             gemm_input_role=gemm_input_role)
 
@@ -86,6 +90,7 @@ class _ToFloat8ConstrFunc(torch.autograd.Function):
         return g, None, None, None, None, None, None
 
 
+@torch._dynamo.allow_in_graph
 class _FromFloat8ConstrFunc(torch.autograd.Function):
     """Float8Tensor -> high precision; the gradient passes through unchanged (reference :198-212)."""
 

@@ -7,6 +7,7 @@ from typing import Iterable, Literal, Tuple, Union
 
 import torch
 
+from . import _custom_ops  # noqa: F401  (registers torch.ops.f8mi.*)
 from . import _native
 from . import config as _config
 
@@ -71,7 +72,8 @@ def tensor_to_amax(x: torch.Tensor, reduce_amax: bool = False) -> torch.Tensor:
     so with an initialised process group of more than one rank it raises.
     """
     _no_multi_rank(reduce_amax)
-    amax, _ = _native.amax_scale(x, e4m3_dtype, want_scale=False)
+    _native._require_gpu(x, "x")
+    amax, _ = torch.ops.f8mi.amax_scale(x, e4m3_dtype, x.dtype, x.dtype == torch.float16)
     return amax.to(x.dtype)  # exact: the maximum is one of x's values
 
 
@@ -80,15 +82,18 @@ def tensor_to_scale(x: torch.Tensor, float8_dtype: torch.dtype, reduce_amax: boo
     """Dynamic scale of x: one pass, amax and scale arithmetic in one kernel (reference :115-120)."""
     _check_fp8(float8_dtype)
     _no_multi_rank(reduce_amax)
-    _, scale = _native.amax_scale(x, float8_dtype, want_amax=False)
+    _native._require_gpu(x, "x")
+    # through the custom op (one opaque node for torch.compile; the same launch in eager mode)
+    _, scale = torch.ops.f8mi.amax_scale(x, float8_dtype, x.dtype, x.dtype == torch.float16)
     return scale
 
 
 def to_fp8_saturated(x: torch.Tensor, float8_dtype: torch.dtype) -> torch.Tensor:
     """clamp to the fp8 range, then convert (reference float8_utils.py:123-139)."""
     _check_fp8(float8_dtype)
+    _native._require_gpu(x, "x")
     one = torch.ones((), dtype=torch.float32, device=x.device)
-    out, _ = _native.cast(x, one, float8_dtype, product_dtype=x.dtype)
+    out, _ = torch.ops.f8mi.cast(x, one, float8_dtype, x.dtype, False)
     return out
 
 

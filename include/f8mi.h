@@ -67,7 +67,10 @@ size_t f8mi_workspace_bytes(void);
  * amax = max|x| and the fp8 scale derived from it, in one pass over x.
  * Replaces tensor_to_amax (float8_utils.py:102-112) + amax_to_scale
  * (float8_utils.py:35-57), i.e. tensor_to_scale (float8_utils.py:115-120).
- *   x          rows x cols elements of `in_dtype`, row stride `ld` elements
+ *   x          rows x cols elements of `in_dtype`, row stride `ld` elements (ld >= cols), or ld = 0: every row is
+ *              the same `cols` elements -- a broadcast row, as autograd hands an expanded gradient
+ *              (float8_scaling_utils.py:204-216 receives y.sum().backward()'s dY that way); f8mi_cast and
+ *              f8mi_cast_dynamic take ld = 0 likewise, and only `cols` elements are read
  *   math_dtype dtype each step of `fmax / clamp(amax, 1e-12)` is rounded to:
  *              `in_dtype` for dynamic scaling (the reference computes the scale
  *              in the tensor's dtype), F8MI_FP32 for delayed-scaling buffers

@@ -293,6 +293,43 @@ def test_cfg1_dy_ones(nat):
     assert bool((out.view(torch.uint8) == 0x7B).all()) and bool((out_t.view(torch.uint8) == 0x7B).all())
 
 
+@pytest.mark.parametrize("shape,strides", [((2048, 4096), (0, 0)), ((2048, 4096), (0, 1)), ((4, 300, 1000), (0, 0, 1)),
+                                           ((40, 512), (0, 1))])
+def test_expanded_gradient_is_cast_without_being_materialised(nat, shape, strides):
+    """dY of ``y.sum().backward()`` is an expanded tensor (reference float8_scaling_utils.py:204-216 casts it like any
+    other): amax, scale and bytes equal those of the materialised tensor, and the binding passes one row with row
+    stride 0 instead of copying rows x cols elements."""
+    torch.manual_seed(9)
+    cols = shape[-1]
+    base = (torch.ones(1, device=DEV) if strides[-1] == 0 else torch.randn(cols, device=DEV) * 0.3).to(torch.bfloat16)
+    dy = torch.as_strided(base, shape, strides)
+    full = dy.contiguous()
+    read, rows, c, ld = nat._as_2d(dy)
+    assert ld == 0 and read.numel() == cols and rows * c == full.numel()
+    for f8, kb in ((torch.float8_e5m2, False), (torch.float8_e4m3fn, True)):
+        kb = kb and cols % 64 == 0 and rows % 64 == 0
+        a0, s0 = nat.amax_scale(full, f8)
+        a1, s1 = nat.amax_scale(dy, f8)
+        assert a0.item() == a1.item() and s0.item() == s1.item()
+        o0, t0 = nat.cast(full.reshape(rows, cols), s0, f8, want_out_t=True, out_kblock=kb, out_t_kblock=kb)
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        before = torch.cuda.memory_allocated()
+        o1, t1 = nat.cast(dy.reshape(rows, cols) if dy.dim() > 2 else dy, s1, f8, want_out_t=True, out_kblock=kb, out_t_kblock=kb)
+        torch.cuda.synchronize()
+        assert torch.cuda.max_memory_allocated() - before < 2 * full.numel() + (1 << 20)  # the two fp8 outputs, no bf16 copy
+        assert torch.equal(o0.view(torch.uint8), o1.view(torch.uint8)) and torch.equal(t0.view(torch.uint8), t1.view(torch.uint8))
+        o2, _, s2 = nat.cast_dynamic(dy.reshape(rows, cols) if dy.dim() > 2 else dy, f8, out_kblock=kb)
+        assert s2.item() == s0.item() and torch.equal(o2.view(torch.uint8), o0.view(torch.uint8))
+        amax = torch.zeros(1, device=DEV)
+        one = torch.ones(1, device=DEV)
+        nat.cast(dy, one, f8, product_dtype=torch.float32, amax_out=amax)  # the delayed-scaling cast records the amax
+        assert amax.item() == a0.item()
+    if strides[-1] == 0:  # dY = ones: scale 57344, every e5m2 byte 0x7B
+        o, _, s = nat.cast_dynamic(dy, torch.float8_e5m2)
+        assert s.item() == 57344.0 and bool((o.view(torch.uint8) == 0x7B).all())
+
+
 def test_golden_cast_fixtures_on_gpu(nat):
     from tests.helpers import from_bits, load
 

@@ -84,8 +84,8 @@ def test_golden_trajectory(f8, name, scaling, hist, steps, dt, emulate):
                 for field, attr in (("amax", "fp8_amax_"), ("hist", "fp8_amax_history_"), ("scale", "fp8_scale_")):
                     got = getattr(lay, attr + kind).cpu().numpy()
                     want = g[f"{tag}.L{li}.{field}_{kind}"]
-                    if (li, kind) in downstream:
-                        np.testing.assert_allclose(got, want, rtol=2e-2, err_msg=str((name, tag, li, field, kind)))
+                    if (li, kind) in downstream:  # one bf16 ulp of the tensor the amax was taken of
+                        np.testing.assert_allclose(got, want, rtol=2.0**-7, err_msg=str((name, tag, li, field, kind)))
                     else:
                         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (name, tag, li, field, kind, got, want)
 
@@ -103,7 +103,7 @@ def test_golden_trajectory(f8, name, scaling, hist, steps, dt, emulate):
             check_buffers(f"t{t}.after")
         for key, val in (("y", y), ("dx", x.grad), ("dw0", model[0].weight.grad), ("db0", model[0].bias.grad),
                          ("dw1", model[1].weight.grad)):
-            _gemm_close(val, from_bits(g[f"t{t}.{key}"], dt), 2e-2, (name, t, key))
+            _gemm_close(val, from_bits(g[f"t{t}.{key}"], dt), 1e-2, (name, t, key))
 
 
 # ------------------------------------------------- all combos vs the oracle

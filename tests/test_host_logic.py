@@ -242,3 +242,54 @@ def test_padding_helpers():
     p = pad_tensor_for_matmul(torch.ones(3, 41).to(torch.float8_e4m3fn), dims=1)
     assert p.shape == (3, 48) and p.dtype == torch.float8_e4m3fn and bool((p.view(torch.uint8)[:, 41:] == 0).all())
     assert is_row_major((8, 1)) and not is_row_major((1, 8))
+
+
+def test_emulated_mm_is_registered_as_an_aten_op():
+    """Schema and Meta implementation of torch.ops.aten.mm_float8_emulated (reference float8_aten_api.py:37-49);
+    no CPU kernel is registered: this package computes on the GPU only."""
+    import float8_experimental_amd  # noqa: F401
+
+    op = torch.ops.aten.mm_float8_emulated.default
+    assert str(op._schema) == "aten::mm_float8_emulated(Tensor m1, Tensor s1, Tensor m2, Tensor s2, ScalarType dtype3) -> Tensor"
+    m1 = torch.empty(5, 7, dtype=torch.float8_e4m3fn, device="meta")
+    m2 = torch.empty(7, 3, dtype=torch.float8_e5m2, device="meta")
+    s = torch.empty((), device="meta")
+    out = op(m1, s, m2, s, torch.bfloat16)
+    assert out.shape == (5, 3) and out.dtype == torch.bfloat16 and out.device.type == "meta"
+    with pytest.raises(NotImplementedError):
+        op(torch.zeros(2, 2).to(torch.float8_e4m3fn), torch.ones(()), torch.zeros(2, 2).to(torch.float8_e4m3fn), torch.ones(()), torch.float32)
+
+
+def test_primitive_custom_ops_have_fake_implementations():
+    """f8mi::amax_scale / cast / gemm_nt trace with fake tensors (shapes and dtypes only, no GPU)."""
+    import float8_experimental_amd  # noqa: F401
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        x = torch.empty(6, 10, 32, dtype=torch.bfloat16, device="cuda")
+        amax, scale = torch.ops.f8mi.amax_scale(x, torch.float8_e4m3fn, torch.bfloat16, False)
+        assert amax.shape == () and scale.shape == () and scale.dtype == torch.float32
+        bits, a = torch.ops.f8mi.cast(x, scale, torch.float8_e5m2, torch.bfloat16, True)
+        assert bits.shape == x.shape and bits.dtype == torch.float8_e5m2 and a.shape == (1,)
+        bits, a = torch.ops.f8mi.cast(x, scale, torch.float8_e4m3fn, torch.float32, False)
+        assert a.numel() == 0
+        a8 = torch.empty(12, 64, dtype=torch.float8_e4m3fn, device="cuda")
+        b8 = torch.empty(20, 64, dtype=torch.float8_e4m3fn, device="cuda")
+        y = torch.ops.f8mi.gemm_nt(a8, scale, b8, scale, torch.float16, None)
+        assert y.shape == (12, 20) and y.dtype == torch.float16
+
+
+def test_get_float8_layers_marks_buffers_static():
+    """Reference float8_linear_utils.py:157-169: buffers of the delayed-scaling layers are marked as static addresses."""
+    import float8_experimental_amd as f8
+
+    cfg = f8.Float8LinearConfig(cast_config_input=f8.CastConfig(f8.ScalingType.DELAYED))
+    model = torch.nn.Sequential(torch.nn.Linear(8, 8), torch.nn.ReLU(), torch.nn.Linear(8, 8))
+    f8.convert_to_float8_training(model, config=cfg)
+    layers = f8.float8_linear_utils.get_float8_layers(model)
+    assert len(layers) == 2
+    for layer in layers:
+        bufs = list(layer.buffers())
+        assert len(bufs) == 9
+        for buf in bufs:
+            assert getattr(buf, "_dynamo_static_input_type", None) == "guarded"
