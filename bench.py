@@ -29,11 +29,89 @@ M_TOKENS = 16384
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
-# Bytes per GEMM launch that cross the L2 boundary (fetch + write), averaged over the 12 launches of a step:
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this script, each scaled by the same counter's reading for a
-# 1 GiB device copy (x2.0 and x1.0); the summary is profiles/bench_llama70b_gemm_hbm_traffic_pmc.txt.
-# Only meaningful at the default --m.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 5.74e9
+# Bytes per GEMM launch that cross the L2 boundary (fetch + write), averaged over the 12 launches of a step, come
+# from a tracked record of the last rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (each counter scaled
+# by its reading for a 1 GiB device copy), which also names the commit and the workload it was measured at.
+GEMM_TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "bench_llama70b_gemm_hbm_traffic.json")
+
+
+def gemm_traffic(m, scaling):
+    """(bytes per GEMM launch past the L2, provenance string) from the tracked profile record; (None, why) when the
+    record is missing or was measured on another workload than this run's."""
+    try:
+        with open(GEMM_TRAFFIC_RECORD) as f:
+            rec = json.load(f)
+    except (OSError, ValueError) as e:
+        return None, f"no record ({type(e).__name__})"
+    if rec.get("m_tokens") != m or rec.get("scaling") != scaling:
+        return None, f"record is for M={rec.get('m_tokens')}, {rec.get('scaling')} scaling"
+    total = rec["fetch_bytes_per_launch"] + rec["write_bytes_per_launch"]
+    why = (f"bytes past the L2 per launch: FETCH_SIZE {rec['fetch_bytes_per_launch']:.4g} + WRITE_SIZE "
+           f"{rec['write_bytes_per_launch']:.4g} (rocprofv3 --pmc, calibrated on a 1 GiB copy), measured at commit "
+           f"{rec.get('commit', '?')} ({os.path.basename(GEMM_TRAFFIC_RECORD)}); algorithmic: "
+           f"{rec.get('algorithmic_bytes_per_launch', 1.035e9):.4g}")
+    return total, why
+
+
+class Telemetry:
+    """Socket power and shader clock of the GPU while the timed region runs, sampled from sysfs by a host thread
+    (reads of two small files every 5 ms; nothing on the launch path)."""
+
+    def __init__(self, period=0.005):
+        import glob
+        import threading
+
+        self.period = period
+        self.power_w, self.sclk_mhz = [], []
+        self.cap_w = None
+        self._stop = threading.Event()
+        self._thread = None
+        self.power_file = self.sclk_file = None
+        for dev in sorted(glob.glob("/sys/class/drm/card[0-9]*/device")):
+            hw = sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*", "power1_input"))
+                        + glob.glob(os.path.join(dev, "hwmon", "hwmon*", "power1_average")))
+            if hw and os.path.exists(os.path.join(dev, "pp_dpm_sclk")):
+                self.power_file, self.sclk_file = hw[0], os.path.join(dev, "pp_dpm_sclk")
+                try:
+                    self.cap_w = int(open(os.path.join(os.path.dirname(hw[0]), "power1_cap")).read()) / 1e6
+                except (OSError, ValueError):
+                    pass
+                break
+
+    def _sample(self):
+        try:
+            self.power_w.append(int(open(self.power_file).read()) / 1e6)
+            for line in open(self.sclk_file).read().splitlines():
+                if line.rstrip().endswith("*"):  # the current level, e.g. "S: 1795Mhz *"
+                    self.sclk_mhz.append(float(line.split(":")[1].strip().split("M")[0]))
+        except (OSError, ValueError, IndexError):
+            pass
+
+    def _run(self):
+        while not self._stop.is_set():
+            self._sample()
+            self._stop.wait(self.period)
+
+    def start(self):
+        import threading
+
+        if self.power_file is None:
+            return
+        self._thread = threading.Thread(target=self._run, daemon=True)
+        self._thread.start()
+
+    def stop(self):
+        self._stop.set()
+        if self._thread is not None:
+            self._thread.join()
+        if not self.power_w:
+            return None
+        mean = lambda v: sum(v) / len(v) if v else None
+        return {"source": "sysfs hwmon power1_input + pp_dpm_sclk, every %d ms over the timed region" % int(self.period * 1e3),
+                "samples": len(self.power_w), "socket_power_W_mean": mean(self.power_w), "socket_power_W_max": max(self.power_w),
+                "power_cap_W": self.cap_w, "sclk_MHz_mean": mean(self.sclk_mhz),
+                "sclk_MHz_min": min(self.sclk_mhz) if self.sclk_mhz else None,
+                "sclk_MHz_max": max(self.sclk_mhz) if self.sclk_mhz else None}
 
 
 def parse():
@@ -185,11 +263,14 @@ def main():
     torch.cuda.synchronize()
     _native.prof_reset()
     _native.prof_enable(True)
+    telemetry = Telemetry()
+    telemetry.start()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step(layers, sync=sync)
     torch.cuda.synchronize()
     sec_step = (time.perf_counter() - t0) / args.steps
+    telemetry = telemetry.stop()
     _native.prof_enable(False)
     prof = {name: _native.prof_read(kid) for name, kid in
             (("amax", _native.K_AMAX), ("cast", _native.K_CAST), ("gemm", _native.K_GEMM))}
@@ -203,6 +284,13 @@ def main():
         hbm[kname] = {"launches": cnt, "GB/s": nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0,
                       "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS if ms > 0 else 0.0,
                       "avg_ms": ms / max(cnt, 1), "algorithmic_GB_per_launch": nbytes / max(cnt, 1) / 1e9}
+
+    if prof["amax"][1] > 0 and prof["cast"][1] > 0:  # dynamic scaling reads every tensor twice: both passes together
+        both_bytes, both_ms = prof["amax"][2] + prof["cast"][2], prof["amax"][1] + prof["cast"][1]
+        hbm["amax_plus_cast"] = {"GB/s": both_bytes / (both_ms * 1e-3) / 1e9,
+                                 "frac_of_hbm_peak": both_bytes / (both_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                 "ms_per_step": both_ms / args.steps}
+    traffic, traffic_note = gemm_traffic(m, args.scaling)
 
     # ---- per shape, and bf16 nn.Linear on the same GPU
     per_shape = {}
@@ -220,6 +308,40 @@ def main():
             per_shape[name]["bf16_TFLOP/s"] = flop_per_shape[name] / t / 1e12
             per_shape[name]["speedup_vs_bf16"] = per_shape[name]["bf16_ms"] / per_shape[name]["fp8_ms"]
         bf16_step = sum(v["bf16_ms"] for v in per_shape.values()) * 1e-3
+
+    # ---- the twelve GEMMs of a step alone, back to back on operands cast beforehand (untimed for `value`): what the
+    # matrix-core kernel sustains, and the socket power and shader clock it runs at, without the cast phases in between
+    gemm_loop = None
+    if args.scaling == "dynamic":
+        E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+        ops = []
+        for name, k, n, lin, mod, x, dy in layers:
+            x8, _, sx = _native.cast_dynamic(x.detach(), E4, out_kblock=True)
+            w8, _, sw = _native.cast_dynamic(lin.weight.detach(), E4, out_kblock=True)
+            g8, _, sg = _native.cast_dynamic(dy, E5, out_kblock=True)
+            ops.append((x8, sx, w8, sw, g8, sg))
+
+        def gemms():
+            for x8, sx, w8, sw, g8, sg in ops:
+                if _native.tn_ok(m, x8.shape[0] * _native.KB, w8.shape[1]):
+                    _native.gemm_nt_kb(x8, sx, w8, sw, torch.bfloat16)
+                    _native.gemm_kb_ex(g8, False, sg, w8, True, sw, torch.bfloat16)
+                    _native.gemm_kb_ex(g8, True, sg, x8, True, sx, torch.bfloat16)
+
+        if all(_native.tn_ok(m, k, n) for _, k, n, *_ in layers):
+            gemms()
+            torch.cuda.synchronize()
+            tele = Telemetry()
+            tele.start()
+            iters = max(8, 2 * args.steps)
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                gemms()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / iters
+            gemm_loop = {"TFLOP/s": flop_step / dt / 1e12, "frac_of_fp8_peak": flop_step / dt / 1e12 / PEAK_FP8_TFLOPS,
+                         "ms_per_12_gemms": dt * 1e3, "iterations": iters, "telemetry": tele.stop()}
+        del ops
 
     # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
     mfma_zero = probe_mfma(torch, False)
@@ -251,15 +373,17 @@ def main():
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_tflops / PEAK_FP8_TFLOPS,
-            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if m == M_TOKENS else None,
-            "traffic_unit": "bytes past the L2 per launch (FETCH_SIZE + WRITE_SIZE, calibrated); algorithmic: 1.035e9",
+            "traffic": traffic,
+            "traffic_unit": traffic_note,
             "launches": n_gemm,
             "avg_launch_ms": ms_gemm / max(n_gemm, 1),
             "flop_per_launch": flop_gemm / max(n_gemm, 1),
             "mfma_only_zero_operands_TFLOP/s": mfma_zero,
             "mfma_only_random_operands_TFLOP/s": mfma_random,
             "frac_of_mfma_only_random": gemm_tflops / mfma_random if mfma_random else None,
+            "gemms_back_to_back": gemm_loop,
         },
+        "telemetry": telemetry,
         "hbm_kernels": hbm,
         "per_shape": per_shape,
         "frac_of_fp8_peak_end_to_end": flop_step / sec_step / 1e12 / PEAK_FP8_TFLOPS,

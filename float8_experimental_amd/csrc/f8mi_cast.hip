@@ -147,11 +147,18 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
     // transposed row, instead of one of the two walking through memory with a huge stride.
     int ty, tx;
     {
-        // consecutive workgroup ids go to the 8 XCDs round-robin; re-deal them so that one XCD (one L2)
-        // gets whole groups of neighbouring tiles and can merge their adjacent output segments
+        // Consecutive workgroup ids go to the 8 XCDs round-robin; re-deal them so that one XCD (one L2) gets whole
+        // groups of 64 neighbouring tiles (an 8 x 8 supertile where the tile grid divides evenly) and can merge
+        // their adjacent output segments, while consecutive groups go to consecutive XCDs: the workgroups in flight
+        // on the whole chip then cover ONE contiguous stretch of the tensor that advances through memory.  (Giving
+        // each XCD its own eighth of the tensor instead, eight fronts far apart, measured 5 % slower in the
+        // benchmark step: 5.36 -> 5.63 TB/s; up to 20 % on tensors below 300 MB.)
         int64_t bid = blockIdx.x;
-        const int64_t nb = gridDim.x;
-        if (nb % 8 == 0) bid = (bid % 8) * (nb / 8) + bid / 8;
+        const int64_t nb = gridDim.x, nb_full = nb - nb % 512;  // ids past the last whole round of 8 groups stay
+        if (bid < nb_full) {
+            const int64_t xcd = bid % 8, j = bid / 8;
+            bid = ((j / 64) * 8 + xcd) * 64 + (j % 64);
+        }
         const int64_t band = bid / ((int64_t)CAST_GROUP * tiles_x);
         const int64_t rem = bid - band * CAST_GROUP * tiles_x;
         const int rows_in_band = (int)min((int64_t)CAST_GROUP, tiles_y - band * CAST_GROUP);
