@@ -30,24 +30,34 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    subprocess.run([HIPCC, *FLAGS, "-c", src, "-o", obj], check=True)
+def _compile(src: str, obj_dir: str = OBJ_DIR, defines=()) -> str:
+    obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
+    subprocess.run([HIPCC, *FLAGS, *defines, "-c", src, "-o", obj], check=True)
     return obj
 
 
-def build(verbose: bool = True) -> str:
-    """Always recompiles every source and relinks the shared library."""
-    os.makedirs(OBJ_DIR, exist_ok=True)
+def build(verbose: bool = True, out: str = LIB, defines=()) -> str:
+    """Always recompiles every source and relinks the shared library.  ``out`` / ``defines`` (-DNAME=value flags) make a
+    measurement build beside the shipped one (load it by pointing F8MI_LIB at it); its objects go to their own folder."""
+    obj_dir = OBJ_DIR if out == LIB else os.path.join(OBJ_DIR, os.path.basename(out) + ".objs")
+    os.makedirs(obj_dir, exist_ok=True)
     srcs = sources()
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
-    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], check=True)
-    subprocess.run([HIPCC, *FLAGS, "-shared", PROBE_SRC, "-o", PROBE_LIB], check=True)
+        objs = list(ex.map(lambda src: _compile(src, obj_dir, tuple(defines)), srcs))
+    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs], check=True)
+    if out == LIB:
+        subprocess.run([HIPCC, *FLAGS, "-shared", PROBE_SRC, "-o", PROBE_LIB], check=True)
     if verbose:
-        print(f"built {LIB} from {len(srcs)} sources", file=sys.stderr)
-    return LIB
+        print(f"built {out} from {len(srcs)} sources", file=sys.stderr)
+    return out
 
 
 if __name__ == "__main__":
-    build()
+    import argparse
+
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--out", default=LIB, help="path of the shared library to write (default: the in-tree libf8mi.so)")
+    ap.add_argument("-D", dest="defines", action="append", default=[], metavar="NAME=value",
+                    help="preprocessor definition for a measurement build, e.g. -DF8MI_WALK_GROUP=2")
+    a = ap.parse_args()
+    build(out=os.path.abspath(a.out), defines=["-D" + d for d in a.defines])

@@ -229,24 +229,17 @@ int cu_count() {
 
 using namespace f8mi;
 
-extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt,
-                               int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
-                               void* stream_) {
-    hipStream_t stream = (hipStream_t)stream_;
-    if (rows < 0 || cols < 0 || (ld < cols && ld != 0)) { set_error("f8mi_amax_scale: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
-    if (in_dtype < 0 || in_dtype > 2 || math_dtype < 0 || math_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_amax_scale: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
-    if (!amax_dev && !scale_dev) { set_error("f8mi_amax_scale: no output requested"); return F8MI_ERR_INVALID_ARG; }
+namespace f8mi {
+
+// First half of f8mi_amax_scale: per-workgroup maxima of the |x| bit patterns into ws[0 .. *nblocks).  rows * cols > 0,
+// arguments already validated.  The second half is amax_finalize_kernel -- or the consumer reduces the words itself
+// (the dynamic-scaling cast does: one launch less).
+int launch_amax_partials(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, uint32_t* ws, hipStream_t stream,
+                         int* nblocks) {
     if (ld == 0 && rows > 1) rows = 1;  // every row is the same `cols` elements: the maximum of one of them
     const int64_t n = rows * cols;
-    if (n == 0) {
-        hipLaunchKernelGGL(amax_empty_kernel, dim3(1), dim3(64), 0, stream, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
-        return check_hip(hipGetLastError(), "amax_empty_kernel");
-    }
-    if (!x || !workspace) { set_error("f8mi_amax_scale: null tensor or workspace"); return F8MI_ERR_INVALID_ARG; }
-    uint32_t* ws = (uint32_t*)workspace;
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
     const bool dense = (ld == cols || rows == 1) && ((uintptr_t)x % 16 == 0);
-    ProfScope prof(F8MI_K_AMAX, (double)n * esz, stream);
     int64_t blocks;
     if (dense) {
         const int64_t epv = 16 / esz;
@@ -270,9 +263,29 @@ extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_
         else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP16>, g, b, 0, stream, x, rows, cols, ld, ws);
         else hipLaunchKernelGGL(amax_strided_kernel<F8MI_FP32>, g, b, 0, stream, x, rows, cols, ld, ws);
     }
-    int rc = check_hip(hipGetLastError(), "amax kernel launch");
-    if (rc) return rc;
-    hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(AMAX_THREADS), 0, stream, ws, (int)blocks, amax_dev, scale_dev, in_dtype,
+    *nblocks = (int)blocks;
+    return check_hip(hipGetLastError(), "amax kernel launch");
+}
+
+}  // namespace f8mi
+
+extern "C" int f8mi_amax_scale(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt,
+                               int math_dtype, int orig_is_fp16, float* amax_dev, float* scale_dev, void* workspace,
+                               void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (rows < 0 || cols < 0 || (ld < cols && ld != 0)) { set_error("f8mi_amax_scale: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
+    if (in_dtype < 0 || in_dtype > 2 || math_dtype < 0 || math_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_amax_scale: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
+    if (!amax_dev && !scale_dev) { set_error("f8mi_amax_scale: no output requested"); return F8MI_ERR_INVALID_ARG; }
+    if (rows * cols == 0) {
+        hipLaunchKernelGGL(amax_empty_kernel, dim3(1), dim3(64), 0, stream, amax_dev, scale_dev, math_dtype, fp8_fmt, orig_is_fp16);
+        return check_hip(hipGetLastError(), "amax_empty_kernel");
+    }
+    if (!x || !workspace) { set_error("f8mi_amax_scale: null tensor or workspace"); return F8MI_ERR_INVALID_ARG; }
+    uint32_t* ws = (uint32_t*)workspace;
+    int blocks = 0;
+    ProfScope prof(F8MI_K_AMAX, (double)(ld == 0 ? cols : rows * cols) * (in_dtype == F8MI_FP32 ? 4 : 2), stream);
+    if (int rc = launch_amax_partials(x, rows, cols, ld, in_dtype, ws, stream, &blocks)) return rc;
+    hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(AMAX_THREADS), 0, stream, ws, blocks, amax_dev, scale_dev, in_dtype,
                        math_dtype, fp8_fmt, orig_is_fp16);
     return check_hip(hipGetLastError(), "amax finalize kernel launch");
 }

@@ -135,9 +135,11 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
                                                             int64_t ld, const float* __restrict__ scale_dev,
                                                             uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
                                                             float* amax_out, int64_t tiles_x, int64_t tiles_y,
-                                                            int out_kb, int out_t_kb) {
+                                                            int out_kb, int out_t_kb, const uint32_t* __restrict__ amax_ws,
+                                                            int amax_nblocks, float* scale_out) {
     __shared__ uint32_t tileT[CAST_TILE * CAST_TILE / 4];  // [column][row/4] dwords, swizzled
     __shared__ uint32_t red[CAST_THREADS / 64];
+    __shared__ uint32_t ws_max;
 
     const int t = threadIdx.x;
     const int a = t & 15;   // column group: columns 8a .. 8a+7 of the tile
@@ -172,13 +174,45 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
     const int64_t c0 = (int64_t)tx * CAST_TILE;
     const int64_t col = c0 + 8 * a;
 
+    // dynamic scaling: this lane's share of the amax kernel's per-workgroup maxima (WS_WORDS = 4 x 256 at most),
+    // requested ahead of the tile so that they arrive first
+    static_assert(WS_WORDS <= 4 * CAST_THREADS, "four words per lane cover the workspace");
+    uint32_t ws_words[4] = {0u, 0u, 0u, 0u};
+    if (amax_ws) {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (t + q * CAST_THREADS < amax_nblocks) ws_words[q] = amax_ws[t + q * CAST_THREADS];
+    }
+
     Row8<DT> in[2][4];
 #pragma unroll
     for (int h = 0; h < 2; h++)
 #pragma unroll
         for (int j = 0; j < 4; j++) load_row8<DT, VEC>(in[h][j], x, r0 + 64 * h + 4 * b + j, col, rows, cols, ld);
 
-    const float scale = *scale_dev;
+    // The scale: given -- or, for dynamic scaling, derived here from the per-workgroup maxima the amax kernel left in
+    // amax_ws (every workgroup reduces the <= 1024 words itself; saves the one-block launch that would do it once).
+    // The words were requested before the tile, and the two barriers wait for LDS only, so the reduction runs while
+    // the tile's loads are still in flight.  Same arithmetic as amax_finalize_kernel, in the tensor's dtype.
+    float scale;
+    if (amax_ws) {
+        uint32_t wm = ws_words[0] > ws_words[1] ? ws_words[0] : ws_words[1];
+        const uint32_t wm2 = ws_words[2] > ws_words[3] ? ws_words[2] : ws_words[3];
+        wm = wave_max_u32(wm > wm2 ? wm : wm2);
+        if ((t & 63) == 0) red[t >> 6] = wm;
+        lds_barrier();
+        if (t == 0) {
+            uint32_t v = red[0];
+#pragma unroll
+            for (int w = 1; w < CAST_THREADS / 64; w++) v = v > red[w] ? v : red[w];
+            ws_max = v;
+        }
+        lds_barrier();
+        scale = amax_to_scale_dev(abs_bits_to_float(ws_max, DT), DT, FMT, DT == F8MI_FP16);
+        if (blockIdx.x == 0 && t == 0) *scale_out = scale;
+    } else {
+        scale = *scale_dev;
+    }
     constexpr float fmax = FMT == F8MI_E4M3FN ? 448.0f : 57344.0f;
 
     uint32_t m = 0;
@@ -351,34 +385,48 @@ static int launch_cast_small(int fmt, bool vec, hipStream_t stream, const void* 
     return check_hip(hipGetLastError(), "cast (dynamic, one workgroup) kernel launch");
 }
 
+// where a dynamic-scaling cast takes its scale from (see cast_layout_impl)
+struct AmaxSource {
+    const uint32_t* ws;
+    int nblocks;
+    float* scale_out;
+};
+
 __global__ void cast_zero_amax_kernel(float* amax_out) {
     if (threadIdx.x == 0) *amax_out = 0.0f;
 }
 
 template <int DT, int PROD, int FMT>
 static int launch_cast2(bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
-                        const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb) {
-    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
-    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+                        const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb,
+                        const AmaxSource& src) {
+    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src.ws, src.nblocks, src.scale_out);
+    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src.ws, src.nblocks, src.scale_out);
     return check_hip(hipGetLastError(), "cast kernel launch");
 }
 
 template <int DT, int PROD>
 static int launch_cast1(int fmt, bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols,
                         int64_t ld, const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev,
-                        int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb) {
-    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
-    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+                        int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb, const AmaxSource& src) {
+    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
 }
+
+// Validates and launches the cast.  `src.ws` null: the scale is read from scale_dev (f8mi_cast_layout).  Not null
+// (dynamic scaling, product in the input's dtype): the kernel derives the scale from the src.nblocks per-workgroup
+// maxima in src.ws and workgroup 0 stores it to src.scale_out.
+static int cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
+                            int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
+                            float* amax_dev, hipStream_t stream, const AmaxSource& src);
 
 }  // namespace f8mi
 
 using namespace f8mi;
 
-extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype,
-                                const float* scale_dev, int product_dtype, int fp8_fmt, uint8_t* out, int out_layout,
-                                uint8_t* out_t, int out_t_layout, float* amax_dev, void* stream_) {
-    hipStream_t stream = (hipStream_t)stream_;
+static int f8mi::cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
+                                  int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
+                                  float* amax_dev, hipStream_t stream, const AmaxSource& src) {
     if ((out_layout != F8MI_LAYOUT_ROWMAJOR && out_layout != F8MI_LAYOUT_KBLOCK64) || (out_t_layout != F8MI_LAYOUT_ROWMAJOR && out_t_layout != F8MI_LAYOUT_KBLOCK64)) { set_error("f8mi_cast: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
     if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
     if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
@@ -387,7 +435,7 @@ extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64
     if (rows < 0 || cols < 0 || (ld < cols && ld != 0)) { set_error("f8mi_cast: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
     if (in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
     if (product_dtype != in_dtype && product_dtype != F8MI_FP32) { set_error("f8mi_cast: product_dtype must be the input dtype or fp32"); return F8MI_ERR_INVALID_ARG; }
-    if (!scale_dev) { set_error("f8mi_cast: null scale"); return F8MI_ERR_INVALID_ARG; }
+    if (!scale_dev && !src.ws) { set_error("f8mi_cast: null scale"); return F8MI_ERR_INVALID_ARG; }
     if (!out && !out_t && !amax_dev) { set_error("f8mi_cast: no output requested"); return F8MI_ERR_INVALID_ARG; }
     if (rows == 0 || cols == 0) {
         if (amax_dev) {
@@ -411,14 +459,21 @@ extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64
     const double n = (double)rows * (double)cols;
     ProfScope prof(F8MI_K_CAST, (ld == 0 ? (double)cols : n) * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
     if (in_dtype == F8MI_BF16) {
-        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
-        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
     }
     if (in_dtype == F8MI_FP16) {
-        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
-        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
     }
-    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb);
+    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+}
+
+extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype,
+                                const float* scale_dev, int product_dtype, int fp8_fmt, uint8_t* out, int out_layout,
+                                uint8_t* out_t, int out_t_layout, float* amax_dev, void* stream) {
+    return cast_layout_impl(x, rows, cols, ld, in_dtype, scale_dev, product_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, amax_dev,
+                            (hipStream_t)stream, AmaxSource{nullptr, 0, nullptr});
 }
 
 extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
@@ -448,9 +503,18 @@ extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int6
         if (in_dtype == F8MI_FP16) return launch_cast_small<F8MI_FP16>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
         return launch_cast_small<F8MI_FP32>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
     }
-    int rc = f8mi_amax_scale(x, rows, cols, ld, in_dtype, fp8_fmt, in_dtype, in_dtype == F8MI_FP16, nullptr, scale_dev, workspace, stream_);
-    if (rc || n == 0 || (!out && !out_t)) return rc;
-    return f8mi_cast_layout(x, rows, cols, ld, in_dtype, scale_dev, in_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, nullptr, stream_);
+    if (n == 0 || (!out && !out_t))  // only the scale is wanted
+        return f8mi_amax_scale(x, rows, cols, ld, in_dtype, fp8_fmt, in_dtype, in_dtype == F8MI_FP16, nullptr, scale_dev, workspace, stream_);
+    if (!x || !workspace) { set_error("f8mi_cast_dynamic: null tensor or workspace"); return F8MI_ERR_INVALID_ARG; }
+    // amax pass: per-workgroup maxima into the workspace; the cast's workgroups reduce them and derive the scale
+    // themselves (no one-block finalize launch in between), workgroup 0 stores it to *scale_dev
+    int nblocks = 0;
+    {
+        ProfScope prof(F8MI_K_AMAX, (double)(ld == 0 ? cols : n) * esz, stream);
+        if (int rc = launch_amax_partials(x, rows, cols, ld, in_dtype, (uint32_t*)workspace, stream, &nblocks)) return rc;
+    }
+    return cast_layout_impl(x, rows, cols, ld, in_dtype, nullptr, in_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, nullptr, stream,
+                            AmaxSource{(const uint32_t*)workspace, nblocks, scale_dev});
 }
 
 namespace f8mi {

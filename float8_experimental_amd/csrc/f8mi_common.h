@@ -28,6 +28,11 @@ struct ProfScope {
 // workspace (uint32 words): one partial max of |x| bit patterns per block of the amax kernel
 constexpr int WS_WORDS = 1024;
 
+// Per-workgroup maxima of the |x| bit patterns into ws[0 .. *nblocks) (f8mi_amax.hip): the first half of
+// f8mi_amax_scale.  rows * cols > 0, arguments already validated; no profiling bracket of its own.
+int launch_amax_partials(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, uint32_t* ws, hipStream_t stream,
+                         int* nblocks);
+
 // ---------------------------------------------------------------- device side
 
 __device__ __forceinline__ float bits_to_float(uint32_t u) { return __uint_as_float(u); }
@@ -130,6 +135,10 @@ __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d)
         return w;
     }
 }
+
+// Workgroup barrier that waits for this wave's LDS traffic only (__syncthreads also waits for every global load
+// the wave has in flight).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 

@@ -7,6 +7,15 @@ namespace f8mi {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// Compile-time knobs of the tile walk, for measurement builds (python _build.py --out other.so -DF8MI_WALK_GROUP=2,
+// loaded through F8MI_LIB); the shipped library is built with the defaults.
+#ifndef F8MI_WALK_GROUP
+#define F8MI_WALK_GROUP 4       // width of the bands the walk sweeps, in tiles
+#endif
+#ifndef F8MI_WALK_XCD_CHUNK
+#define F8MI_WALK_XCD_CHUNK 0   // 0: each XCD owns one contiguous run of the tile order
+#endif
+
 constexpr int SLAB_BYTES = 256 * 128;   // one operand, one step
 constexpr int HALF_BYTES = 256 * 64;    // one 64-deep unit of it
 constexpr int NSLAB_A = 3, NSLAB_B = 2;
@@ -189,11 +198,24 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
     // ---- which tile (same walk as the other kernels)
     int lid = blockIdx.x;
     const int npid = gridDim.x;
+#if F8MI_WALK_XCD_CHUNK == 0
     lid = xcd_contiguous_id(lid, npid);
+#else
+    {   // measurement builds only: chunks of F8MI_WALK_XCD_CHUNK tile ids dealt round-robin to the XCDs
+        const int full = npid - npid % (NUM_XCD * F8MI_WALK_XCD_CHUNK);
+        if (lid < full) {
+            const int x = lid % NUM_XCD, j = lid / NUM_XCD;
+            lid = ((j / F8MI_WALK_XCD_CHUNK) * NUM_XCD + x) * F8MI_WALK_XCD_CHUNK + (j % F8MI_WALK_XCD_CHUNK);
+        }
+    }
+#endif
     // The walk sweeps along the longer side of the tile grid in bands GROUP tiles wide, so that an XCD's 32
     // workgroups hold a 4 x 8 (or 8 x 4) patch of neighbouring tiles; sweeping along the shorter side instead
     // cost 1 - 3 % on the shapes where the sides differ most (measured both ways on all twelve benchmark GEMMs).
-    constexpr int GROUP = 4;
+    // Per 128-deep step such a patch pulls 4 + 8 operand panels through the XCD's L2 for 32 tiles, the least that 32
+    // tiles in step allow; bytes fetched past the L2 and GEMM rate by band width, same box, benchmark step: 1 tile
+    // 14.2 GB per launch / 2982 TFLOP/s, 2 tiles 7.8 / 3190, 4 tiles 5.2 / 3250, 8 tiles 5.2 / 3259, 16 tiles - / 3187.
+    constexpr int GROUP = F8MI_WALK_GROUP;
     int tm, tn;
     if (tiles_m > tiles_n) {
         const int width = GROUP * tiles_m;

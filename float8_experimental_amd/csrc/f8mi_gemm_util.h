@@ -29,9 +29,6 @@ __device__ __forceinline__ int xcd_contiguous_id(int bid, int grid) {
 
 #define F8MI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-// Workgroup barrier that waits for this wave's LDS traffic only.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
 __device__ __forceinline__ v8i read_frag(const uint8_t* p0, const uint8_t* p1) {
     const uint4 lo = *(const uint4*)p0;
     const uint4 hi = *(const uint4*)p1;
