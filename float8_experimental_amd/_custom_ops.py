@@ -34,7 +34,8 @@ def amax_scale(x: torch.Tensor, float8_dtype: torch.dtype, math_dtype: torch.dty
         torch.Tensor, torch.Tensor]:
     """(max|x|, fp8 scale of it), both 0-dim fp32, in one pass over x: ``tensor_to_amax`` + ``amax_to_scale`` of the
     reference (float8_utils.py:35-57, 102-120) with the scale arithmetic rounded to ``math_dtype``."""
-    return _native.amax_scale(x, float8_dtype, math_dtype=math_dtype, orig_is_fp16=orig_is_fp16)
+    with _native.transient_workspaces():
+        return _native.amax_scale(x, float8_dtype, math_dtype=math_dtype, orig_is_fp16=orig_is_fp16)
 
 
 @amax_scale.register_fake
@@ -64,7 +65,8 @@ def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: t
             bias: Optional[torch.Tensor]) -> torch.Tensor:
     """``(a @ bt^T) / (a_scale * b_scale) (+ bias)`` on the matrix cores: ``torch._scaled_mm`` as the reference calls it
     (float8_python_api.py:24-64), with the second operand given as [n, k]."""
-    return _native.gemm_nt(a, a_scale, bt, b_scale, out_dtype, bias=bias)
+    with _native.transient_workspaces():
+        return _native.gemm_nt(a, a_scale, bt, b_scale, out_dtype, bias=bias)
 
 
 @gemm_nt.register_fake
@@ -109,6 +111,11 @@ def linear_fwd(x2: torch.Tensor, weight: torch.Tensor, need_dx: bool, need_dw: b
     and one that backward will not need is an empty tensor.  sx / sw are the scales of dynamically scaled
     tensors; for a tensor with delayed scaling (``scale_*`` given: the module's scale buffer) the slot holds an empty
     tensor and ``amax_*`` this step's amax, [1] fp32 (empty for dynamic scaling)."""
+    with _native.transient_workspaces():
+        return _linear_fwd_impl(x2, weight, need_dx, need_dw, scale_x, scale_w)
+
+
+def _linear_fwd_impl(x2, weight, need_dx, need_dw, scale_x, scale_w):
     m, k = x2.shape
     n = weight.shape[0]
     none = lambda dt: torch.empty(0, dtype=dt, device=x2.device)
@@ -146,6 +153,11 @@ def linear_bwd(dy2: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, sx: torch.
         torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dx, dw, amax_g): (dY W, dY^T x) in fp8, dY cast to e5m2 with a dynamic scale or the delayed-scaling scale
     buffer (then amax_g is this step's amax of dY, [1] fp32; else empty); an unneeded gradient is empty."""
+    with _native.transient_workspaces():
+        return _linear_bwd_impl(dy2, xs, ws, sx, sw, k, need_dx, need_dw, scale_g)
+
+
+def _linear_bwd_impl(dy2, xs, ws, sx, sw, k, need_dx, need_dw, scale_g):
     m, n = dy2.shape
     empty = lambda: torch.empty(0, dtype=dy2.dtype, device=dy2.device)
     if _native.tn_ok(m, k, n):
@@ -219,9 +231,10 @@ def sync(amaxes: List[torch.Tensor], histories: List[torch.Tensor], scales: List
     """The delayed-scaling sync of all listed buffers as one node (and one kernel launch): for each i,
     ``scales[i] = fmax / max(amaxes[i], histories[i][:-1])`` in the reference's rounding
     (float8_linear_utils.py:287-319).  No autograd: the buffers carry none."""
-    table = _native.sync_table_cached((a, h, s, e5m2_dtype if e else e4m3_dtype)
-                                      for a, h, s, e in zip(amaxes, histories, scales, is_e5m2))
-    _native.sync(table, histories[0].numel(), orig_is_fp16, writeback_history=False)
+    # the entries travel as kernel arguments: a node of a compiled graph must not allocate a tensor that outlives it
+    # (torch.compile(mode="reduce-overhead") keeps the graph's memory in a pool of its own)
+    _native.sync_host(((a, h, s, e5m2_dtype if e else e4m3_dtype) for a, h, s, e in zip(amaxes, histories, scales, is_e5m2)),
+                      histories[0].numel(), orig_is_fp16, writeback_history=False)
 
 
 @sync.register_fake

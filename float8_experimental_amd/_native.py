@@ -42,6 +42,7 @@ EXPORTS = (
     "f8mi_gemm_nt_kb",
     "f8mi_gemm_kb_ex",
     "f8mi_sync",
+    "f8mi_sync_host",
     "f8mi_delayed_init",
     "f8mi_prof_enable",
     "f8mi_prof_reset",
@@ -107,6 +108,8 @@ def lib() -> C.CDLL:
         L.f8mi_gemm_nt_kb_ws.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp, i64, vp]
         L.f8mi_sync.restype = i32
         L.f8mi_sync.argtypes = [vp, i32, i32, i32, i32, vp]
+        L.f8mi_sync_host.restype = i32
+        L.f8mi_sync_host.argtypes = [vp, i32, i32, i32, i32, vp]
         L.f8mi_delayed_init.restype = i32
         L.f8mi_delayed_init.argtypes = [fp, fp, fp, i32, i32, i32, vp]
         L.f8mi_prof_enable.restype = i32
@@ -162,11 +165,30 @@ def _check_device(dev: torch.device) -> None:
 
 
 _workspaces = {}
+_tls = threading.local()
+
+
+class transient_workspaces:
+    """While active (per thread), ``workspace`` and ``gemm_workspace`` hand out fresh tensors instead of the cached
+    per-(device, stream) ones.  The custom ops that ``torch.compile`` calls run under it: a node of a compiled graph must
+    not leave a tensor of its own behind in the graph's memory pool (``mode="reduce-overhead"`` checks that), while a
+    temporary that dies with the call is fine -- the allocator hands its memory out again in stream order."""
+
+    def __enter__(self):
+        self.prev = getattr(_tls, "transient", False)
+        _tls.transient = True
+
+    def __exit__(self, *exc):
+        _tls.transient = self.prev
+        if not self.prev:
+            _tls.gemm_ws = None  # the kernels that use it are already queued; its memory is reused in stream order
 
 
 def workspace(dev: torch.device) -> torch.Tensor:
     """Reduction workspace of f8mi_amax_scale (per-block partial maxima), one per (device, stream)."""
     _check_device(dev)
+    if getattr(_tls, "transient", False):
+        return torch.empty(lib().f8mi_workspace_bytes() // 4, dtype=torch.int32, device=dev)
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), _raw_stream(dev))
     ws = _workspaces.get(key)
     if ws is None:
@@ -180,12 +202,18 @@ _GEMM_WS_MIN_ROWS, _GEMM_WS_MIN_K = 17, 2048  # below these no GEMM is ever spli
 _gemm_workspaces = {}
 
 
-def gemm_workspace(dev: torch.device, m: int, k: int):
+def gemm_workspace(dev: torch.device, m: int, k: int, n: int = 0):
     """(pointer, bytes) of the scratch that lets a few-row GEMM with a long contraction split k over workgroups; one
     allocation per (device, stream), made the first time a shape that could use it comes by; (None, 0) for shapes
     that never do."""
     if m < _GEMM_WS_MIN_ROWS or k < _GEMM_WS_MIN_K:
         return None, 0
+    if getattr(_tls, "transient", False):
+        # a temporary, and only for a product the library would actually split over k
+        if (lib().f8mi_gemm_plan(m, n, k, 1, GEMM_WORKSPACE_BYTES) & 0xff) != 1:
+            return None, 0
+        _tls.gemm_ws = torch.empty(GEMM_WORKSPACE_BYTES // 4, dtype=torch.float32, device=dev)
+        return _tls.gemm_ws.data_ptr(), GEMM_WORKSPACE_BYTES
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), _raw_stream(dev))
     ws = _gemm_workspaces.get(key)
     if ws is None:
@@ -431,7 +459,7 @@ def gemm_nt_kb(a_kb: torch.Tensor, a_scale: torch.Tensor, bt_kb: torch.Tensor, b
     if bias is not None:
         assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a_kb.device
     _check_device(a_kb.device)
-    ws, ws_bytes = gemm_workspace(a_kb.device, m, k) if split_k else (None, 0)
+    ws, ws_bytes = gemm_workspace(a_kb.device, m, k, n) if split_k else (None, 0)
     rc = lib().f8mi_gemm_nt_kb_ws(a_kb.data_ptr(), _F8[a_kb.dtype], bt_kb.data_ptr(), _F8[bt_kb.dtype], m, n, k,
                                   a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
                                   bias.data_ptr() if bias is not None else None, ws, ws_bytes, _stream(a_kb))
@@ -499,7 +527,7 @@ def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: t
     if bias is not None:
         assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a.device
     _check_device(a.device)
-    ws, ws_bytes = gemm_workspace(a.device, m, k) if split_k else (None, 0)
+    ws, ws_bytes = gemm_workspace(a.device, m, k, n) if split_k else (None, 0)
     rc = lib().f8mi_gemm_nt_ws(a.data_ptr(), _F8[a.dtype], lda, bt.data_ptr(), _F8[bt.dtype], ldb, m, n, k,
                                a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], max(n, 1),
                                bias.data_ptr() if bias is not None else None, ws, ws_bytes, _stream(a))
@@ -541,6 +569,26 @@ def sync(table: torch.Tensor, hist_len: int, orig_is_fp16: bool, writeback_histo
     rc = lib().f8mi_sync(table.data_ptr(), table.shape[0], hist_len, int(orig_is_fp16), int(writeback_history),
                          _stream(table))
     _check(rc, "f8mi_sync")
+
+
+def sync_host(entries, hist_len: int, orig_is_fp16: bool, writeback_history: bool = False) -> None:
+    """``sync`` without a device table: ``entries`` (iterable of (amax, history, scale, float8_dtype)) go to the GPU as
+    kernel arguments.  Allocates no tensor, which is what a compiled graph with its own memory pool needs."""
+    rows = []
+    dev = None
+    for amax, hist, scale, f8 in entries:
+        for t in (amax, hist, scale):
+            _require_gpu(t, "buffer")
+            assert t.dtype == torch.float32 and t.is_contiguous()
+        assert hist.numel() == hist_len
+        rows += [amax.data_ptr(), hist.data_ptr(), scale.data_ptr(), _F8[f8]]
+        dev = amax.device
+    if not rows:
+        return
+    _check_device(dev)
+    arr = (C.c_int64 * len(rows))(*rows)
+    rc = lib().f8mi_sync_host(arr, len(rows) // 4, hist_len, int(orig_is_fp16), int(writeback_history), _raw_stream(dev))
+    _check(rc, "f8mi_sync_host")
 
 
 def delayed_init(amax: torch.Tensor, history: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype,

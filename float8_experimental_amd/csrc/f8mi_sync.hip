@@ -5,11 +5,7 @@
 
 namespace f8mi {
 
-__global__ void sync_kernel(const f8mi_sync_entry* __restrict__ entries, int n, int hist_len, int orig_is_fp16,
-                            int writeback) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const f8mi_sync_entry e = entries[i];
+__device__ __forceinline__ void sync_entry(const f8mi_sync_entry& e, int hist_len, int orig_is_fp16, int writeback) {
     const float amax = *e.amax;
     // S = roll(history, 1); S[0] = amax  ->  max(S) = max(amax, history[0 .. H-2])
     float mx = amax;
@@ -25,6 +21,26 @@ __global__ void sync_kernel(const f8mi_sync_entry* __restrict__ entries, int n, 
         e.history[0] = amax;
     }
     *e.scale = amax_to_scale_dev(mx, F8MI_FP32, (int)e.fp8_fmt, orig_is_fp16);
+}
+
+__global__ void sync_kernel(const f8mi_sync_entry* __restrict__ entries, int n, int hist_len, int orig_is_fp16,
+                            int writeback) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    sync_entry(entries[i], hist_len, orig_is_fp16, writeback);
+}
+
+// The same with the entries passed by value as a kernel argument (no table in device memory to build, copy or
+// keep): SYNC_CHUNK entries per launch.
+constexpr int SYNC_CHUNK = 32;
+struct SyncChunk {
+    f8mi_sync_entry e[SYNC_CHUNK];
+};
+
+__global__ void sync_args_kernel(SyncChunk chunk, int n, int hist_len, int orig_is_fp16, int writeback) {
+    const int i = threadIdx.x;
+    if (blockIdx.x != 0 || i >= n) return;
+    sync_entry(chunk.e[i], hist_len, orig_is_fp16, writeback);
 }
 
 __global__ void delayed_init_kernel(const float* amax_dev, float* history, float* scale, int hist_len, int fmt,
@@ -58,6 +74,28 @@ extern "C" int f8mi_sync(const f8mi_sync_entry* entries_dev, int n, int hist_len
     hipLaunchKernelGGL(sync_kernel, dim3((n + threads - 1) / threads), dim3(threads), 0, stream, entries_dev, n,
                        hist_len, orig_is_fp16, writeback_history);
     return check_hip(hipGetLastError(), "sync_kernel launch");
+}
+
+extern "C" int f8mi_sync_host(const f8mi_sync_entry* entries_host, int n, int hist_len, int orig_is_fp16,
+                              int writeback_history, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n < 0 || hist_len < 1) { set_error("f8mi_sync_host: bad n=%d or hist_len=%d", n, hist_len); return F8MI_ERR_INVALID_ARG; }
+    if (n == 0) return F8MI_OK;
+    if (!entries_host) { set_error("f8mi_sync_host: null entry array"); return F8MI_ERR_INVALID_ARG; }
+    for (int i = 0; i < n; i++)
+        if (!entries_host[i].amax || !entries_host[i].history || !entries_host[i].scale || entries_host[i].fp8_fmt < 0 || entries_host[i].fp8_fmt > 1) {
+            set_error("f8mi_sync_host: entry %d has a null pointer or an unknown fp8 format", i);
+            return F8MI_ERR_INVALID_ARG;
+        }
+    ProfScope prof(F8MI_K_SYNC, (double)n * (hist_len + 2) * 4.0, stream);
+    for (int first = 0; first < n; first += SYNC_CHUNK) {
+        SyncChunk chunk = {};
+        const int m = n - first < SYNC_CHUNK ? n - first : SYNC_CHUNK;
+        for (int i = 0; i < m; i++) chunk.e[i] = entries_host[first + i];
+        hipLaunchKernelGGL(sync_args_kernel, dim3(1), dim3(64), 0, stream, chunk, m, hist_len, orig_is_fp16, writeback_history);
+        if (int rc = check_hip(hipGetLastError(), "sync_args_kernel launch")) return rc;
+    }
+    return F8MI_OK;
 }
 
 extern "C" int f8mi_delayed_init(const float* amax_dev, float* history_dev, float* scale_dev, int hist_len,

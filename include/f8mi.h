@@ -265,6 +265,14 @@ typedef struct f8mi_sync_entry {
 int f8mi_sync(const f8mi_sync_entry* entries_dev, int n, int hist_len, int orig_is_fp16, int writeback_history,
               void* stream);
 
+/* f8mi_sync with the entries in HOST memory: they travel to the GPU by value, as kernel arguments, 32 per launch, so
+ * there is no table in device memory to build, copy or keep alive.  For callers whose device allocations are managed
+ * by someone else -- a compiled graph under torch.compile(mode="reduce-overhead") must not keep a tensor of its own
+ * inside the graph's memory pool -- and for one-off calls.  Under stream capture the pointers are baked into the
+ * captured launches: the buffers must stay where they are (as for any captured kernel). */
+int f8mi_sync_host(const f8mi_sync_entry* entries_host, int n, int hist_len, int orig_is_fp16, int writeback_history,
+                   void* stream);
+
 /*
  * First-iteration initialisation of one tensor's buffers
  * (_maybe_initialize_amaxes_scales_for_float8_cast, float8_scaling_utils.py:99-125):

@@ -62,6 +62,11 @@ def test_host_side_argument_checks_need_no_gpu():
     assert rc == -1
     rc = lib.f8mi_sync(None, -1, 16, 0, 0, None)
     assert rc == -1
+    rc = lib.f8mi_sync_host(None, 3, 16, 0, 0, None)
+    assert rc == -1
+    bad = (ctypes.c_int64 * 4)(8, 0, 8, 0)  # null history pointer
+    rc = lib.f8mi_sync_host(bad, 1, 16, 0, 0, None)
+    assert rc == -1 and b"entry 0" in lib.f8mi_last_error()
     # k-blocked operands: k must be a multiple of 64 and at least 384 (unsupported, not invalid)
     rc = lib.f8mi_gemm_nt_kb(None, 0, None, 0, i64(4), i64(4), i64(100), None, None, None, 0, i64(4), None, None)
     assert rc == -2 and b"k-blocked" in lib.f8mi_last_error()

@@ -164,6 +164,64 @@ def test_sync_compiles_into_one_frame(f8, backend):
     assert all(m.amax_and_scale_synced is False for m in f8.float8_linear_utils.get_float8_layers(b))  # post-forward ran
 
 
+def test_sync_under_cudagraphs_is_not_skipped(f8):
+    """Reference: test_compile.py:294-320 -- torch.compile(sync, mode="reduce-overhead") must really run as a
+    captured graph: get_float8_layers marks the buffers as static addresses, so the mutation of the scale buffers by
+    the sync node is no reason to skip.  The replays are compared with an eager twin, with eager work in between."""
+    from torch._dynamo.utils import counters
+
+    _need_inductor()
+    torch.manual_seed(8)
+    D = f8.CastConfig(f8.ScalingType.DELAYED)
+    cfg = f8.Float8LinearConfig(cast_config_input=D, cast_config_weight=D, cast_config_grad_output=D)
+    base = nn.Sequential(nn.Linear(16, 32, bias=True), nn.ReLU(), nn.Linear(32, 16, bias=True)).to(DEV)
+    a, b = copy.deepcopy(base), copy.deepcopy(base)
+    f8.convert_to_float8_training(a, config=cfg)
+    f8.convert_to_float8_training(b, config=cfg)
+    torch._dynamo.reset()
+    counters.clear()
+    sync_func = torch.compile(f8.sync_float8_amax_and_scale_history, mode="reduce-overhead", fullgraph=True)
+    layers_b = f8.float8_linear_utils.get_float8_layers(b)
+    for it in range(5):
+        x = torch.randn(16, 16, device=DEV) * 2.0 ** it
+        dy = torch.randn(16, 16, device=DEV)
+        for u, v in zip(_run(b, x, dy), _run(a, x, dy)):  # eager steps: record amaxes, clear the synced flag
+            assert torch.equal(u, v), it
+        f8.sync_float8_amax_and_scale_history(a)
+        sync_func(b, layers_b)
+        for (name, b1), (_, b2) in zip(a.named_buffers(), b.named_buffers()):
+            assert torch.equal(b1, b2), (it, name)
+    assert counters["inductor"]["cudagraph_skips"] == 0, dict(counters["inductor"])
+
+
+@pytest.mark.parametrize("shape,n", [((64, 512), 448), ((3, 768, 2048), 2432)])
+def test_model_under_cudagraphs(f8, shape, n):
+    """torch.compile(model, mode="reduce-overhead"): forward and backward are captured graphs that replay the library's
+    kernels.  The custom ops leave nothing of their own in the graph's memory pool (their workspaces are temporaries
+    there), so nothing is skipped; every replay gives the bits of the eager run."""
+    from torch._dynamo.utils import counters
+
+    _need_inductor()
+    torch.manual_seed(9)
+    k = shape[-1]
+    base = nn.Sequential(nn.Linear(k, n, bias=False), nn.Linear(n, 384, bias=False)).to(DEV, dtype=torch.bfloat16)
+    a, b = copy.deepcopy(base), copy.deepcopy(base)
+    f8.convert_to_float8_training(a)
+    f8.convert_to_float8_training(b)
+    torch._dynamo.reset()
+    counters.clear()
+    cb = torch.compile(b, mode="reduce-overhead", fullgraph=True)
+    for it in range(5):  # warm-up, capture, then replays, with the eager twin's work in between
+        x = torch.randn(shape, device=DEV, dtype=torch.bfloat16) * 1.5 ** it
+        dy = torch.randn(*shape[:-1], 384, device=DEV, dtype=torch.bfloat16)
+        want = _run(a, x, dy)
+        got = [t.clone() for t in _run(cb, x, dy)]
+        torch.cuda.synchronize()
+        for u, v in zip(got, want):
+            assert torch.equal(u, v), it
+    assert counters["inductor"]["cudagraph_skips"] == 0, dict(counters["inductor"])
+
+
 def test_whole_delayed_scaling_step_as_one_graph(f8):
     """sync + forward in one compiled function: the scales the sync node writes are the ones the casts read."""
     torch.manual_seed(6)
