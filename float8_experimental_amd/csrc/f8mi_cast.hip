@@ -418,15 +418,7 @@ static int launch_cast1(int fmt, bool vec, dim3 g, hipStream_t stream, const voi
 // maxima in src.ws and workgroup 0 stores it to src.scale_out.
 static int cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
                             int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
-                            float* amax_dev, hipStream_t stream, const AmaxSource& src);
-
-}  // namespace f8mi
-
-using namespace f8mi;
-
-static int f8mi::cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
-                                  int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
-                                  float* amax_dev, hipStream_t stream, const AmaxSource& src) {
+                            float* amax_dev, hipStream_t stream, const AmaxSource& src) {
     if ((out_layout != F8MI_LAYOUT_ROWMAJOR && out_layout != F8MI_LAYOUT_KBLOCK64) || (out_t_layout != F8MI_LAYOUT_ROWMAJOR && out_t_layout != F8MI_LAYOUT_KBLOCK64)) { set_error("f8mi_cast: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
     if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
     if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
@@ -468,6 +460,10 @@ static int f8mi::cast_layout_impl(const void* x, int64_t rows, int64_t cols, int
     }
     return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
 }
+
+}  // namespace f8mi
+
+using namespace f8mi;
 
 extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype,
                                 const float* scale_dev, int product_dtype, int fp8_fmt, uint8_t* out, int out_layout,
