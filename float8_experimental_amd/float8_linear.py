@@ -332,15 +332,20 @@ class Float8Linear(torch.nn.Linear):
 
     def _forward_under_compile(self, input: torch.Tensor) -> torch.Tensor:
         """What ``torch.compile`` traces: one custom-op node per direction (plus the bias add), with the delayed-scaling
-        buffers as arguments the node writes.  Anything that keeps Python state -- the first-iteration amax
-        initialisation, the pre/post-forward flags (``enable_amax_init`` / ``enable_pre_and_post_forward``: switch both
-        off for a graph without breaks, as with the reference) -- or carries Float8Tensors runs outside the graph."""
+        buffers as arguments the node writes -- or, for ``emulate=True`` and pre-cast operands, the reference's op-by-op
+        composition.  Anything that keeps Python state -- the first-iteration amax initialisation, the pre/post-forward
+        flags (``enable_amax_init`` / ``enable_pre_and_post_forward``: switch both off for a graph without breaks, as
+        with the reference) -- runs outside the graph."""
         stateless = (not self.has_any_delayed_scaling
                      or (self.is_amax_initialized and not self.enable_pre_and_post_forward))
-        plain = (stateless and not self.config.emulate and self._precomputed_weight_scale is None
+        if not stateless:
+            return self._forward_outside_graph(input)
+        plain = (not self.config.emulate and self._precomputed_weight_scale is None
                  and not isinstance(self.weight, Float8Tensor) and not isinstance(input, Float8Tensor))
         if not plain:
-            return self._forward_outside_graph(input)
+            # emulate=True, a precomputed weight scale, operands that are Float8Tensors already: the reference's own
+            # composition, whose pieces (casts, the matmul of two Float8Tensors, the emulated aten op) are opaque nodes
+            return self._forward_composed_body(input)
         from ._custom_ops import linear
 
         def bufs(kind):

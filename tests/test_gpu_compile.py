@@ -522,6 +522,48 @@ def test_compiled_delayed_scaling_against_the_oracle(f8, backend, scaling):
             assert err <= 1e-2, (it, key, err)
 
 
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+@pytest.mark.parametrize("scaling", [("dyn", "dyn", "dyn"), ("del", "del", "del")])
+def test_compiled_emulate_true_against_the_oracle(f8, backend, scaling):
+    """emulate=True under fullgraph=True (reference test_compile.py: emulate in {True, False}): the module traces as the
+    reference's own composition -- casts, matmul of two Float8Tensors, aten::mm_float8_emulated -- and the oracle IS that
+    arithmetic: scales bit-exact, outputs to the summation order of an fp32 matmul (one ulp of bf16)."""
+    from oracle import torch_oracle as to
+
+    m = {"dyn": f8.ScalingType.DYNAMIC, "del": f8.ScalingType.DELAYED}
+    cfg = f8.Float8LinearConfig(cast_config_input=f8.CastConfig(m[scaling[0]]), cast_config_weight=f8.CastConfig(m[scaling[1]]),
+                                cast_config_grad_output=f8.CastConfig(m[scaling[2]]), emulate=True,
+                                enable_amax_init=False, enable_pre_and_post_forward=False)
+    torch.manual_seed(17)
+    lin = nn.Linear(128, 96, bias=True).to(torch.bfloat16)
+    mod = f8.Float8Linear.from_float(copy.deepcopy(lin), config=cfg).to(DEV)
+    orc = to.LinearOracle(lin.weight.detach().clone(), scaling, 16)
+    orc.is_amax_initialized = True
+    orc.last_seen_input_dtype = torch.bfloat16
+    torch._dynamo.reset()
+    cm = torch.compile(mod, backend=_backend(backend), fullgraph=True)
+    for it in range(3):
+        x = (torch.randn(4, 16, 128) * 1.4 ** it).to(torch.bfloat16)
+        dy = (torch.randn(4, 16, 96) * 0.05).to(torch.bfloat16)
+        if "del" in scaling:
+            f8.sync_float8_amax_and_scale_history(mod)
+            orc.sync()
+        xd = x.to(DEV).requires_grad_()
+        mod.weight.grad = None
+        mod.bias.grad = None
+        y = cm(xd)
+        y.backward(dy.to(DEV))
+        ref = orc.fwd_bwd(x, dy)
+        if scaling[0] == "del":
+            assert mod.fp8_amax_input.cpu().item() == orc.st["input"].amax.item(), it
+            assert mod.fp8_amax_grad_output.cpu().item() == orc.st["grad_output"].amax.item(), it
+        want_y = (ref["y"].float() + lin.bias.float()).to(torch.bfloat16)
+        for key, val, want in (("y", y, want_y), ("dx", xd.grad, ref["dx"]), ("dw", mod.weight.grad, ref["dw"])):
+            want = want.float()
+            torch.testing.assert_close(val.detach().float().cpu(), want, rtol=2.0**-7, atol=2.0**-8 * want.abs().max().item(),
+                                       msg=lambda msg: f"{key} it={it}: {msg}")
+
+
 def test_emulated_mm_is_an_aten_op(f8):
     """torch.ops.aten.mm_float8_emulated (reference float8_aten_api.py:37-49) against the oracle's restatement."""
     from oracle import torch_oracle as to
