@@ -162,7 +162,7 @@ def sha(t):
 
 
 def cfg1():
-    """BASELINE config 1: one dynamic fwd+bwd of Linear(4096,4096) on x[2048,4096], seed 0."""
+    """Benchmark configuration 1: one dynamic fwd+bwd of Linear(4096,4096) on x[2048,4096], seed 0."""
     torch.manual_seed(0)
     lin = nn.Linear(4096, 4096, bias=False).to(torch.bfloat16)
     x = torch.randn(2048, 4096).to(torch.bfloat16).requires_grad_()

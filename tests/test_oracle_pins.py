@@ -138,7 +138,7 @@ def test_scale_known_answers():
     # fp16: EPS rounds to 0, 1/0 = inf, clamp to 65504 (reference test_base.py:566-586)
     assert co.amax_to_scale(0.0, co.FP16, co.E4M3FN, True) == 65504.0
     assert np.isnan(co.amax_to_scale(np.nan, co.BF16, co.E4M3FN))
-    # dY = ones (BASELINE config 1): scale 57344, every byte 0x7B
+    # dY = ones (benchmark configuration 1): scale 57344, every byte 0x7B
     assert co.cast(np.full((2, 4), 0x3F80, np.uint16), co.BF16, 57344.0, co.BF16, co.E5M2)[0].tolist() == [[0x7B] * 4] * 2
 
 
