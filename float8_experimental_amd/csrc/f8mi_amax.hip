@@ -15,6 +15,24 @@ namespace f8mi {
 constexpr int AMAX_THREADS = 256;
 constexpr int AMAX_UNROLL = 8;  // 16-byte loads in flight per thread
 
+// Loads are non-temporal.  Measurement builds can read tensors of up to F8MI_AMAX_PLAIN_LOADS_MAX_BYTES with ordinary
+// loads instead (-DF8MI_AMAX_PLAIN_LOADS_MAX_BYTES=...), which leave the tensor in the 256 MB memory-side cache for
+// the cast that follows.  Measured in the benchmark step (kernel times from a trace, amax + cast of one tensor):
+//   every tensor with ordinary loads: 134 MB 59.7 -> 55.7 us, 168 MB 72.5 -> 71.6, but 268 MB 111.6 -> 121.4,
+//     470 MB 199.5 -> 238.4, 1.9 GB 774 -> 816 (the cast gains 3 - 10 %, the amax pass loses 30 - 70 %);
+//   only tensors up to 192 MB with ordinary loads: 134 MB 59.7 -> 66.9 us, 168 MB 72.5 -> 80.9 -- worse than either.
+// A line allocated in that cache pushes out a line that is there, and when that is a dirty line -- the fp8 copy or the
+// GEMM output written just before -- its write-back competes with the reads: what ordinary loads cost depends on what
+// the kernels before left in the cache, not on the tensor's size, and no size rule survives a change of neighbours.
+#ifndef F8MI_AMAX_PLAIN_LOADS_MAX_BYTES
+#define F8MI_AMAX_PLAIN_LOADS_MAX_BYTES 0
+#endif
+template <bool NT>
+__device__ __forceinline__ uint4 amax_load16(const uint4* p) {
+    if constexpr (NT) return load_nt16(p);
+    else return *p;
+}
+
 // sign-cleared patterns of the elements packed in one 32-bit word, reduced to one value
 template <int DT>
 __device__ __forceinline__ uint32_t absmax_word(uint32_t w) {
@@ -76,7 +94,7 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_finalize_kernel(const uint3
 // 16-byte vectors (32 KB of contiguous memory); inside a tile consecutive lanes read consecutive
 // vectors, so every wave-level load is 1 KB of one DRAM page.  (Striding each lane's loads by the whole
 // grid instead costs more than half of the bandwidth.)
-template <int DT>
+template <int DT, bool NT>
 __global__ __launch_bounds__(AMAX_THREADS) void amax_dense_kernel(const void* __restrict__ x, int64_t n,
                                                                    uint32_t* __restrict__ ws) {
     __shared__ uint32_t red[AMAX_THREADS / 64];
@@ -91,12 +109,12 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_dense_kernel(const void* __
         uint4 v[AMAX_UNROLL];
         if (base - threadIdx.x + TILE <= nvec) {
 #pragma unroll
-            for (int u = 0; u < AMAX_UNROLL; u++) v[u] = load_nt16(&xv[base + u * AMAX_THREADS]);
+            for (int u = 0; u < AMAX_UNROLL; u++) v[u] = amax_load16<NT>(&xv[base + u * AMAX_THREADS]);
         } else {
 #pragma unroll
             for (int u = 0; u < AMAX_UNROLL; u++) {
                 const int64_t i = base + u * AMAX_THREADS;
-                v[u] = i < nvec ? load_nt16(&xv[i]) : make_uint4(0, 0, 0, 0);
+                v[u] = i < nvec ? amax_load16<NT>(&xv[i]) : make_uint4(0, 0, 0, 0);
             }
         }
 #pragma unroll
@@ -250,9 +268,17 @@ int launch_amax_partials(const void* x, int64_t rows, int64_t cols, int64_t ld, 
         if (blocks > cap) blocks = cap;
         if (blocks < 1) blocks = 1;
         dim3 g((unsigned)blocks), b(AMAX_THREADS);
-        if (in_dtype == F8MI_BF16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_BF16>, g, b, 0, stream, x, n, ws);
-        else if (in_dtype == F8MI_FP16) hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP16>, g, b, 0, stream, x, n, ws);
-        else hipLaunchKernelGGL(amax_dense_kernel<F8MI_FP32>, g, b, 0, stream, x, n, ws);
+        const bool nt = (int64_t)(n * esz) > (int64_t)F8MI_AMAX_PLAIN_LOADS_MAX_BYTES;
+        if (in_dtype == F8MI_BF16) {
+            if (nt) hipLaunchKernelGGL((amax_dense_kernel<F8MI_BF16, true>), g, b, 0, stream, x, n, ws);
+            else hipLaunchKernelGGL((amax_dense_kernel<F8MI_BF16, false>), g, b, 0, stream, x, n, ws);
+        } else if (in_dtype == F8MI_FP16) {
+            if (nt) hipLaunchKernelGGL((amax_dense_kernel<F8MI_FP16, true>), g, b, 0, stream, x, n, ws);
+            else hipLaunchKernelGGL((amax_dense_kernel<F8MI_FP16, false>), g, b, 0, stream, x, n, ws);
+        } else {
+            if (nt) hipLaunchKernelGGL((amax_dense_kernel<F8MI_FP32, true>), g, b, 0, stream, x, n, ws);
+            else hipLaunchKernelGGL((amax_dense_kernel<F8MI_FP32, false>), g, b, 0, stream, x, n, ws);
+        }
     } else {
         blocks = (n + AMAX_THREADS - 1) / AMAX_THREADS;
         int64_t cap = (int64_t)cu_count() * 8;

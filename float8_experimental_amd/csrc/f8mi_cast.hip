@@ -18,6 +18,10 @@
 
 namespace f8mi {
 
+#ifndef F8MI_CAST_REVERSE_WALK
+#define F8MI_CAST_REVERSE_WALK 0
+#endif
+
 constexpr int CAST_THREADS = 256;
 constexpr int CAST_TILE = 128;
 constexpr int CAST_GROUP = 8;
@@ -161,6 +165,9 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
             const int64_t xcd = bid % 8, j = bid / 8;
             bid = ((j / 64) * 8 + xcd) * 64 + (j % 64);
         }
+#if F8MI_CAST_REVERSE_WALK  // measurement builds only: last tiles first, the reverse of the order the amax pass read in
+        bid = nb - 1 - bid;
+#endif
         const int64_t band = bid / ((int64_t)CAST_GROUP * tiles_x);
         const int64_t rem = bid - band * CAST_GROUP * tiles_x;
         const int rows_in_band = (int)min((int64_t)CAST_GROUP, tiles_y - band * CAST_GROUP);
