@@ -33,25 +33,24 @@ __device__ __forceinline__ uint4 amax_load16(const uint4* p) {
     else return *p;
 }
 
-// sign-cleared patterns of the elements packed in one 32-bit word, reduced to one value
-template <int DT>
-__device__ __forceinline__ uint32_t absmax_word(uint32_t w) {
-    if constexpr (DT == F8MI_FP32) {
-        return w & 0x7fffffffu;
-    } else {
-        uint32_t lo = w & 0x7fffu, hi = (w >> 16) & 0x7fffu;
-        return lo > hi ? lo : hi;
-    }
-}
-
+// Folds the sign-cleared patterns of one 16-byte vector into the running maximum `m`.  16-bit types keep two
+// 16-bit maxima side by side in `m` (absmax16x2) until absmax_done merges them.
 template <int DT>
 __device__ __forceinline__ uint32_t absmax_vec(uint4 v, uint32_t m) {
-    uint32_t a = absmax_word<DT>(v.x), b = absmax_word<DT>(v.y);
-    uint32_t c = absmax_word<DT>(v.z), d = absmax_word<DT>(v.w);
-    a = a > b ? a : b;
-    c = c > d ? c : d;
-    a = a > c ? a : c;
-    return m > a ? m : a;
+    if constexpr (DT == F8MI_FP32) {
+        uint32_t a = v.x & 0x7fffffffu, b = v.y & 0x7fffffffu, c = v.z & 0x7fffffffu, d = v.w & 0x7fffffffu;
+        a = a > b ? a : b;
+        c = c > d ? c : d;
+        a = a > c ? a : c;
+        return m > a ? m : a;
+    } else {
+        return absmax16x2(v.w, absmax16x2(v.z, absmax16x2(v.y, absmax16x2(v.x, m))));
+    }
+}
+template <int DT>
+__device__ __forceinline__ uint32_t absmax_done(uint32_t m) {
+    if constexpr (DT == F8MI_FP32) return m;
+    else return fold16(m);
 }
 
 template <int DT>
@@ -120,6 +119,7 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_dense_kernel(const void* __
 #pragma unroll
         for (int u = 0; u < AMAX_UNROLL; u++) m = absmax_vec<DT>(v[u], m);
     }
+    m = absmax_done<DT>(m);
     if (blockIdx.x == 0) {  // scalar tail (< EPV elements)
         int64_t t = nvec * EPV + threadIdx.x;
         if (t < n) {
@@ -174,13 +174,15 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_multi_kernel(const f8mi_ten
         if (refs[mid].first_tile <= t0) lo = mid; else hi = mid - 1;
     }
     int cur = lo;
-    uint32_t m = 0;
+    uint32_t m = 0, mv = 0;  // maximum of single elements; of whole vectors (two 16-bit maxima side by side, see absmax_vec)
     for (int64_t t = t0; t < t1; t++) {
         while (cur + 1 < n && refs[cur + 1].first_tile <= t) {  // block-uniform: flush and move on
-            m = block_max_u32(m, red);
+            mv = absmax_done<DT>(mv);
+            m = block_max_u32(m > mv ? m : mv, red);
             if (threadIdx.x == 0 && m) atomicMax(&ws[cur], m);
             __syncthreads();
             m = 0;
+            mv = 0;
             cur++;
         }
         const f8mi_tensor_ref r = refs[cur];
@@ -206,9 +208,10 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_multi_kernel(const f8mi_ten
             }
         }
 #pragma unroll
-        for (int u = 0; u < AMAX_UNROLL; u++) m = absmax_vec<DT>(v[u], m);
+        for (int u = 0; u < AMAX_UNROLL; u++) mv = absmax_vec<DT>(v[u], mv);
     }
-    m = block_max_u32(m, red);
+    mv = absmax_done<DT>(mv);
+    m = block_max_u32(m > mv ? m : mv, red);
     if (threadIdx.x == 0 && m) atomicMax(&ws[cur], m);
 }
 

@@ -29,7 +29,9 @@ constexpr int CAST_GROUP = 8;
 // Fused amax of the cast kernel: *amax_out was zeroed by a tiny kernel launched just before, and holds the
 // running maximum as an fp32 bit pattern (non-negative floats and NaNs order like unsigned integers).
 // No ticket and, for all but a handful of blocks, no atomic at all: the value only grows, so a block whose
-// maximum is not above a (possibly stale) read of it has nothing to add.
+// maximum is not above a (possibly stale) read of it has nothing to add.  (Reducing and reading the word early, right
+// after the loads, so that the round trip overlaps the conversion, was 20 % slower: the barrier it needs in the
+// middle of the block makes all four waves wait for the slowest one's loads before any of them converts.)
 __device__ __forceinline__ void publish_amax_cast(uint32_t blockmax, float* amax_out, int in_dt) {
     if (threadIdx.x == 0) {
         const uint32_t bits = __float_as_uint(abs_bits_to_float(blockmax, in_dt));
@@ -89,6 +91,8 @@ __device__ __forceinline__ float elem(const Row8<DT>& r, int i) {
     }
 }
 
+// Folds the eight elements of a row into a running maximum.  16-bit types: `m` holds two 16-bit maxima side by side
+// (see absmax16x2); absmax_done merges them.
 template <int DT>
 __device__ __forceinline__ uint32_t absmax_row(const Row8<DT>& r, uint32_t m) {
     if constexpr (DT == F8MI_FP32) {
@@ -96,13 +100,14 @@ __device__ __forceinline__ uint32_t absmax_row(const Row8<DT>& r, uint32_t m) {
         for (int i = 0; i < 8; i++) { uint32_t a = r.w[i] & 0x7fffffffu; m = m > a ? m : a; }
     } else {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            uint32_t lo = r.w[i] & 0x7fffu, hi = (r.w[i] >> 16) & 0x7fffu;
-            m = m > lo ? m : lo;
-            m = m > hi ? m : hi;
-        }
+        for (int i = 0; i < 4; i++) m = absmax16x2(r.w[i], m);
     }
     return m;
+}
+template <int DT>
+__device__ __forceinline__ uint32_t absmax_done(uint32_t m) {
+    if constexpr (DT == F8MI_FP32) return m;
+    else return fold16(m);
 }
 
 // Loads 8 elements of row `row` starting at column `col`; out-of-range elements read as +0.
@@ -143,7 +148,6 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
                                                             int amax_nblocks, float* scale_out) {
     __shared__ uint32_t tileT[CAST_TILE * CAST_TILE / 4];  // [column][row/4] dwords, swizzled
     __shared__ uint32_t red[CAST_THREADS / 64];
-    __shared__ uint32_t ws_max;
 
     const int t = threadIdx.x;
     const int a = t & 15;   // column group: columns 8a .. 8a+7 of the tile
@@ -181,14 +185,14 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
     const int64_t c0 = (int64_t)tx * CAST_TILE;
     const int64_t col = c0 + 8 * a;
 
-    // dynamic scaling: this lane's share of the amax kernel's per-workgroup maxima (WS_WORDS = 4 x 256 at most),
-    // requested ahead of the tile so that they arrive first
-    static_assert(WS_WORDS <= 4 * CAST_THREADS, "four words per lane cover the workspace");
-    uint32_t ws_words[4] = {0u, 0u, 0u, 0u};
+    // dynamic scaling: the amax kernel's per-workgroup maxima (at most WS_WORDS = 4 x 64 lanes x 4 words), requested
+    // ahead of the tile so that they arrive first.  Every wave fetches all of them: no LDS, no barrier.
+    static_assert(WS_WORDS <= 4 * 64 * 4, "four 16-byte loads per lane cover the workspace");
+    uint4 ws_words[4];
     if (amax_ws) {
 #pragma unroll
         for (int q = 0; q < 4; q++)
-            if (t + q * CAST_THREADS < amax_nblocks) ws_words[q] = amax_ws[t + q * CAST_THREADS];
+            ws_words[q] = q * 256 < amax_nblocks ? ((const uint4*)amax_ws)[q * 64 + (t & 63)] : make_uint4(0u, 0u, 0u, 0u);
     }
 
     Row8<DT> in[2][4];
@@ -198,24 +202,27 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
         for (int j = 0; j < 4; j++) load_row8<DT, VEC>(in[h][j], x, r0 + 64 * h + 4 * b + j, col, rows, cols, ld);
 
     // The scale: given -- or, for dynamic scaling, derived here from the per-workgroup maxima the amax kernel left in
-    // amax_ws (every workgroup reduces the <= 1024 words itself; saves the one-block launch that would do it once).
-    // The words were requested before the tile, and the two barriers wait for LDS only, so the reduction runs while
-    // the tile's loads are still in flight.  Same arithmetic as amax_finalize_kernel, in the tensor's dtype.
+    // amax_ws (every wave of every workgroup reduces the <= 1024 words itself; saves the one-block launch that would do
+    // it once).  The words were requested before the tile and nothing here waits for anybody else, so the reduction
+    // runs while the tile's loads are still in flight.  (A first version shared the work among the four waves through
+    // LDS: its two barriers, in the middle of the block, cost more than the redundant loads do.)  Words past
+    // amax_nblocks are leftovers of an earlier, larger call and are masked.  Same arithmetic as amax_finalize_kernel,
+    // in the tensor's dtype.
     float scale;
     if (amax_ws) {
-        uint32_t wm = ws_words[0] > ws_words[1] ? ws_words[0] : ws_words[1];
-        const uint32_t wm2 = ws_words[2] > ws_words[3] ? ws_words[2] : ws_words[3];
-        wm = wave_max_u32(wm > wm2 ? wm : wm2);
-        if ((t & 63) == 0) red[t >> 6] = wm;
-        lds_barrier();
-        if (t == 0) {
-            uint32_t v = red[0];
+        uint32_t wm = 0;
 #pragma unroll
-            for (int w = 1; w < CAST_THREADS / 64; w++) v = v > red[w] ? v : red[w];
-            ws_max = v;
+        for (int q = 0; q < 4; q++) {
+            const int first = q * 256 + (t & 63) * 4;
+            const uint32_t w[4] = {ws_words[q].x, ws_words[q].y, ws_words[q].z, ws_words[q].w};
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint32_t v = first + c < amax_nblocks ? w[c] : 0u;
+                wm = wm > v ? wm : v;
+            }
         }
-        lds_barrier();
-        scale = amax_to_scale_dev(abs_bits_to_float(ws_max, DT), DT, FMT, DT == F8MI_FP16);
+        wm = wave_max_u32(wm);
+        scale = amax_to_scale_dev(abs_bits_to_float(wm, DT), DT, FMT, DT == F8MI_FP16);
         if (blockIdx.x == 0 && t == 0) *scale_out = scale;
     } else {
         scale = *scale_dev;
@@ -228,6 +235,7 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
         for (int h = 0; h < 2; h++)
 #pragma unroll
             for (int j = 0; j < 4; j++) m = absmax_row<DT>(in[h][j], m);
+        m = absmax_done<DT>(m);
     }
 
     const bool out_vec = (cols % 8 == 0) && ((uintptr_t)out % 8 == 0);
@@ -332,7 +340,7 @@ __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const
     }
 #pragma unroll
     for (int u = 0; u < SMALL_ITEMS_PER_THREAD; u++) m = absmax_row<DT>(r[u], m);
-    m = wave_max_u32(m);
+    m = wave_max_u32(absmax_done<DT>(m));
     if ((t & 63) == 0) red[t >> 6] = m;
     __syncthreads();
     if (t < 64) {
@@ -509,6 +517,11 @@ extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int6
     if (n == 0 || (!out && !out_t))  // only the scale is wanted
         return f8mi_amax_scale(x, rows, cols, ld, in_dtype, fp8_fmt, in_dtype, in_dtype == F8MI_FP16, nullptr, scale_dev, workspace, stream_);
     if (!x || !workspace) { set_error("f8mi_cast_dynamic: null tensor or workspace"); return F8MI_ERR_INVALID_ARG; }
+    if ((uintptr_t)workspace % 16 != 0) {  // the cast reads the workspace in 16-byte pieces: an odd one takes the two calls as they are
+        int rc = f8mi_amax_scale(x, rows, cols, ld, in_dtype, fp8_fmt, in_dtype, in_dtype == F8MI_FP16, nullptr, scale_dev, workspace, stream_);
+        if (rc) return rc;
+        return f8mi_cast_layout(x, rows, cols, ld, in_dtype, scale_dev, in_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, nullptr, stream_);
+    }
     // amax pass: per-workgroup maxima into the workspace; the cast's workgroups reduce them and derive the scale
     // themselves (no one-block finalize launch in between), workgroup 0 stores it to *scale_dev
     int nblocks = 0;

@@ -148,6 +148,18 @@ __device__ __forceinline__ uint4 load_nt16(const void* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// Running maximum of sign-cleared 16-bit patterns, two per dword: `m` holds two independent 16-bit maxima
+// (v_and + v_pk_max_u16 per dword instead of five scalar operations); fold16 merges the halves at the end.
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t absmax16x2(uint32_t w, uint32_t m) {
+    const u16x2 a = __builtin_bit_cast(u16x2, w & 0x7fff7fffu), b = __builtin_bit_cast(u16x2, m);
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+__device__ __forceinline__ uint32_t fold16(uint32_t m) {
+    const uint32_t lo = m & 0xffffu, hi = m >> 16;
+    return lo > hi ? lo : hi;
+}
+
 // wave-wide max of a uint32 (wave64)
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 #pragma unroll
