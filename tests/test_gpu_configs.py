@@ -134,6 +134,38 @@ def test_config2_dynamic_scaling_at_llama70b_shapes(f8, name, k, n):
     # the three products on sampled rows / columns, within 1e-2 of the emulated reference
     _sampled_linear_check(to, x.detach(), w, dy, y.detach(), x.grad, mod.weight.grad, sx, sw, sg, 200 + len(name), f"config2 {name}")
 
+    # ... and EVERY output element through row and column checksums: the sums of a product's rows / columns are a
+    # matrix-vector product of the fp8 operands, evaluated here in fp64 on the device (fp8 values are exact in fp64).
+    # A tile written to the wrong place, left out or computed from the wrong operand block moves a checksum by tens
+    # of per cent of its size; the bf16 rounding of 16384+ summed outputs moves it by a few tenths of a per cent.
+    g8_kb, _, _ = _native.cast_dynamic(dy, E5M2, want_out=True, out_kblock=True)
+    f64 = torch.float64
+    rowmajor = lambda t_kb: t_kb.permute(1, 0, 2).reshape(t_kb.shape[1], -1)
+    xq = rowmajor(x8_kb).to(torch.float32)      # [m, k]
+    wq = rowmajor(w8_kb).to(torch.float32)      # [n, k]
+    gq = rowmajor(g8_kb).to(torch.float32)      # [m, n]
+    del g8_kb
+    sxd, swd, sgd = sx.double().item(), sw.double().item(), sg.double().item()
+
+    def checksums(out, rows_of, cols_of, what):
+        got_c, got_r = out.sum(0, dtype=f64), out.sum(1, dtype=f64)
+        want_c, want_r = cols_of(), rows_of()
+        for got, want, axis in ((got_c, want_c, "column"), (got_r, want_r, "row")):
+            err = (got - want).abs().max().item() / want.abs().max().item()
+            assert err <= 1e-2, (name, what, axis, err)
+
+    matvec = lambda mat, vec: (mat.to(f64) @ vec.to(f64)) if mat.numel() <= (1 << 29) else torch.cat(
+        [c.to(f64) @ vec.to(f64) for c in mat.split(8192)])
+    # y[m, n] = sum_k xq[m, k] wq[n, k] / (sx sw)
+    checksums(y.detach(), lambda: matvec(xq, wq.sum(0, dtype=f64)) / (sxd * swd),
+              lambda: matvec(wq, xq.sum(0, dtype=f64)) / (sxd * swd), "y")
+    # dx[m, k] = sum_n gq[m, n] wq[n, k] / (sg sw)
+    checksums(x.grad, lambda: matvec(gq, wq.sum(1, dtype=f64)) / (sgd * swd),
+              lambda: matvec(wq.t(), gq.sum(0, dtype=f64)) / (sgd * swd), "dx")
+    # dw[n, k] = sum_m gq[m, n] xq[m, k] / (sg sx)
+    checksums(mod.weight.grad, lambda: matvec(gq.t(), xq.sum(1, dtype=f64)) / (sgd * sxd),
+              lambda: matvec(xq.t(), gq.sum(1, dtype=f64)) / (sgd * sxd), "dw")
+
 
 # ------------------------------------------------------------------ config 3
 
