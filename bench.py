@@ -168,9 +168,10 @@ def timed(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def probe_mfma(torch, random_data, iters=4000):
+def probe_mfma(torch, random_data, iters=4000, operands=None):
     """TFLOP/s of a register-only fp8 MFMA loop on every CU: the matrix cores' ceiling with no memory traffic, on zero
-    operands (clock limit) or random ones (power limit).  From libf8mi_probe.so, a bench-only helper next to the library."""
+    operands (clock limit), random ones (power limit) or -- ``operands``: an fp8 tensor of at least 256 KiB -- the bytes
+    of a real tensor.  From libf8mi_probe.so, a bench-only helper next to the library."""
     import ctypes as C
 
     path = os.path.join(ROOT, "float8_experimental_amd", "libf8mi_probe.so")
@@ -180,8 +181,12 @@ def probe_mfma(torch, random_data, iters=4000):
     lib.f8mi_probe_mfma.restype = C.c_int
     lib.f8mi_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_double), C.c_void_p]
     scratch = torch.empty(1 << 20, dtype=torch.uint8, device="cuda:0")
+    mode = int(random_data)
+    if operands is not None:
+        scratch[:1 << 18].copy_(operands.reshape(-1).view(torch.uint8)[:1 << 18])
+        mode = 2
     out = C.c_double(0.0)
-    rc = lib.f8mi_probe_mfma(int(random_data), iters, scratch.data_ptr(), scratch.numel(), C.byref(out),
+    rc = lib.f8mi_probe_mfma(mode, iters, scratch.data_ptr(), scratch.numel(), C.byref(out),
                              torch.cuda.current_stream().cuda_stream)
     return out.value if rc == 0 else None
 
@@ -311,7 +316,7 @@ def main():
 
     # ---- the twelve GEMMs of a step alone, back to back on operands cast beforehand (untimed for `value`): what the
     # matrix-core kernel sustains, and the socket power and shader clock it runs at, without the cast phases in between
-    gemm_loop = None
+    gemm_loop = mfma_real = None
     if args.scaling == "dynamic":
         E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
         ops = []
@@ -341,6 +346,8 @@ def main():
             dt = (time.perf_counter() - t0) / iters
             gemm_loop = {"TFLOP/s": flop_step / dt / 1e12, "frac_of_fp8_peak": flop_step / dt / 1e12 / PEAK_FP8_TFLOPS,
                          "ms_per_12_gemms": dt * 1e3, "iterations": iters, "telemetry": tele.stop()}
+        # the same register-only loop on the fp8 bytes the benchmark's GEMMs actually multiply (x8 of the first shape)
+        mfma_real = probe_mfma(torch, True, operands=ops[0][0])
         del ops
 
     # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
@@ -380,6 +387,7 @@ def main():
             "flop_per_launch": flop_gemm / max(n_gemm, 1),
             "mfma_only_zero_operands_TFLOP/s": mfma_zero,
             "mfma_only_random_operands_TFLOP/s": mfma_random,
+            "mfma_only_benchmark_operands_TFLOP/s": mfma_real,
             "frac_of_mfma_only_random": gemm_tflops / mfma_random if mfma_random else None,
             "gemms_back_to_back": gemm_loop,
         },
