@@ -8,6 +8,7 @@ its epilogue).  The weight stays a ``Float8Tensor`` parameter with row-major byt
 reference keeps it (``inference.py:119-141``), so state dicts interchange; next to it the module
 caches the same bytes in the k-blocked placement the GEMM reads fastest.
 """
+import weakref
 from dataclasses import dataclass
 from enum import Enum, auto
 from typing import Callable, Optional
@@ -15,6 +16,7 @@ from typing import Callable, Optional
 import torch
 import torch.nn as nn
 
+from . import _custom_ops  # noqa: F401  (registers torch.ops.f8mi.*)
 from . import _native
 from .float8_linear_utils import swap_linear_layers
 from .float8_tensor import (
@@ -66,6 +68,58 @@ def _to_kblock(rowmajor_fp8: torch.Tensor) -> torch.Tensor:
     return (rowmajor_fp8.view(torch.uint8).view(rows, k // kb, kb).permute(1, 0, 2).contiguous().view(rowmajor_fp8.dtype))
 
 
+# k-blocked copies of quantised weights, by the address of the row-major bytes; rebuilt when those bytes change
+# (version counter) and dropped with the weight.  Module-level so that the custom op, which sees plain tensors, finds it.
+_KB_WEIGHTS = {}
+
+
+def _kblocked_weight(w_data: torch.Tensor) -> torch.Tensor:
+    key = w_data.data_ptr()
+    tag = (w_data._version, tuple(w_data.shape), w_data.dtype)
+    hit = _KB_WEIGHTS.get(key)
+    if hit is None or hit[0] != tag:
+        if hit is None:
+            weakref.finalize(w_data, _KB_WEIGHTS.pop, key, None)
+        hit = _KB_WEIGHTS[key] = (tag, _to_kblock(w_data))
+    return hit[1]
+
+
+def _fp8_linear(x2: torch.Tensor, w_data: torch.Tensor, w_scale: torch.Tensor, static_scale: Optional[torch.Tensor],
+                bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """x2 [m, k] high precision, w_data [n, k] fp8 row-major -> [m, n] in x2's dtype: activation cast (static scale if
+    given, else dynamic) and the scaled GEMM with the bias in its epilogue."""
+    k = x2.shape[1]
+    use_kb = _native.kblock_ok(k)
+    if static_scale is not None:
+        scale = static_scale
+        x8, _ = _native.cast(x2, scale, e4m3_dtype, product_dtype=_product_dtype(x2, scale), out_kblock=use_kb)
+    else:
+        x8, _, scale = _native.cast_dynamic(x2, e4m3_dtype, out_kblock=use_kb)
+    if use_kb:
+        return _native.gemm_nt_kb(x8, scale, _kblocked_weight(w_data), w_scale, x2.dtype, bias=bias)
+    return _native.gemm_nt(x8, scale, w_data, w_scale, x2.dtype, bias=bias)
+
+
+@torch.library.custom_op("f8mi::inference_linear", mutates_args=())
+def _inference_linear_op(x2: torch.Tensor, w_data: torch.Tensor, w_scale: torch.Tensor, static_scale: Optional[torch.Tensor],
+                         bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``_fp8_linear`` as one opaque node for ``torch.compile`` (workspaces are temporaries inside a compiled graph)."""
+    with _native.transient_workspaces():
+        return _fp8_linear(x2, w_data, w_scale, static_scale, bias)
+
+
+@_inference_linear_op.register_fake
+def _(x2, w_data, w_scale, static_scale, bias):
+    return torch.empty((x2.shape[0], w_data.shape[0]), dtype=x2.dtype, device=x2.device)
+
+
+@torch._dynamo.allow_in_graph
+def _inference_linear_traced(x2: torch.Tensor, weight: "Float8Tensor", static_scale: Optional[torch.Tensor],
+                             bias: Optional[torch.Tensor]) -> torch.Tensor:
+    # taken apart here, below dynamo: the compiler's tracer sees the Float8Tensor's payload and scale as plain tensors
+    return torch.ops.f8mi.inference_linear(x2, weight._data, weight._scale, static_scale, bias)
+
+
 class Float8InferenceLinear(torch.nn.Linear):
     """``nn.Linear`` whose weight is an fp8 ``Float8Tensor`` (``inference.py:70-172`` of the reference)."""
 
@@ -78,19 +132,11 @@ class Float8InferenceLinear(torch.nn.Linear):
             self.register_buffer("static_quantization_scale", quant_config.static_quantization_scale)
         else:
             self.static_quantization_scale = None
-        self._w_kb = None       # k-blocked copy of the weight's bytes, built on first use
-        self._w_kb_key = None
 
     # ---- forward
     def _weight_kblocked(self) -> torch.Tensor:
-        w = self.weight
-        key = (w._data.data_ptr(), w._data._version, tuple(w._data.shape))
-        if self._w_kb is None or self._w_kb_key != key:
-            self._w_kb = _to_kblock(w._data)
-            self._w_kb_key = key
-        return self._w_kb
+        return _kblocked_weight(self.weight._data)
 
-    @torch._dynamo.disable  # the ctypes calls cannot be traced: under torch.compile this module runs outside the graph
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         if self.activation_casting == ActivationCasting.WEIGHT_ONLY:
             # the reference does not pass the bias on this branch either (inference.py:104-107)
@@ -102,22 +148,14 @@ class Float8InferenceLinear(torch.nn.Linear):
             x_fp8 = cast_to_float8_e4m3_inference(input, self.linear_mm_config,
                                                   static_quantization_scale=self.static_quantization_scale)
             return torch.nn.functional.linear(x_fp8, w, self.bias)
-        k = input.shape[-1]
-        x2 = input.reshape(-1, k)
-        out_dtype = input.dtype
+        x2 = input.reshape(-1, input.shape[-1])
         bias = self.bias
-        if bias is not None and bias.dtype != out_dtype:
-            bias = bias.to(out_dtype)
-        use_kb = _native.kblock_ok(k)
-        if self.static_quantization_scale is not None:
-            scale = self.static_quantization_scale
-            x8, _ = _native.cast(x2, scale, e4m3_dtype, product_dtype=_product_dtype(x2, scale), out_kblock=use_kb)
+        if bias is not None and bias.dtype != input.dtype:
+            bias = bias.to(input.dtype)
+        if torch.compiler.is_compiling():  # one opaque node: the ctypes calls cannot be traced
+            y = _inference_linear_traced(x2, w, self.static_quantization_scale, bias)
         else:
-            x8, _, scale = _native.cast_dynamic(x2, e4m3_dtype, out_kblock=use_kb)
-        if use_kb:
-            y = _native.gemm_nt_kb(x8, scale, self._weight_kblocked(), w._scale, out_dtype, bias=bias)
-        else:
-            y = _native.gemm_nt(x8, scale, w._data, w._scale, out_dtype, bias=bias)
+            y = _fp8_linear(x2, w._data, w._scale, self.static_quantization_scale, bias)
         return y.reshape(*input.shape[:-1], self.out_features)
 
     # ---- builders (inference.py:119-172)
@@ -129,12 +167,12 @@ class Float8InferenceLinear(torch.nn.Linear):
                                                          GemmInputRole.WEIGHT)
         self.weight = nn.Parameter(quantized_weight)
         self.weight.requires_grad = False
-        self._w_kb = None
+        if quantized_weight._data.is_cuda and _native.kblock_ok(self.in_features):
+            self._weight_kblocked()  # now, not inside the first forward (which may be a node of a compiled graph)
 
     def set_weight_and_bias(self, weight: torch.nn.Parameter, bias: Optional[torch.nn.Parameter]):
         self.weight = weight
         self.bias = bias
-        self._w_kb = None
 
     @classmethod
     def from_float(cls, module: nn.Module, quant_config: QuantConfig, use_fast_accum: bool) -> "Float8InferenceLinear":

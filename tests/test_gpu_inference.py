@@ -67,6 +67,41 @@ def test_mlp_flows_sqnr(f8, dtype, mode):
     assert _sqnr(f8, want, got) > 20
 
 
+@pytest.mark.parametrize("backend", ["eager", "aot_eager", "inductor"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["dynamic", "static", "weight_only"])
+def test_mlp_flows_compile_fullgraph(f8, backend, dtype, mode):
+    """test_inference_flows.py:60-168 compiles both MLPs with fullgraph=True: the quantised MLP must trace without a
+    break (each fp8 linear is one opaque node) and keep SQNR > 20 dB against the high-precision one; with the eager and
+    aot_eager backends, where the compiler changes no arithmetic of its own, the bits of the uncompiled module."""
+    from float8_experimental_amd.inference import ActivationCasting, QuantConfig, quantize_to_float8
+
+    if backend == "inductor":
+        from tests.test_gpu_compile import _need_inductor
+
+        _need_inductor()
+    torch.manual_seed(1)
+    base = FeedForward(d=1024, ffn=2816, bias=(mode != "weight_only")).to(DEV, dtype=dtype)
+    q = copy.deepcopy(base)
+    cfg = {"dynamic": QuantConfig(ActivationCasting.DYNAMIC),
+           "static": QuantConfig(ActivationCasting.STATIC, static_quantization_scale=torch.tensor([1.0], device=DEV)),
+           "weight_only": QuantConfig(ActivationCasting.WEIGHT_ONLY)}[mode]
+    quantize_to_float8(q, cfg)
+    x = torch.randn(4, 256, 1024, device=DEV, dtype=dtype)
+    torch._dynamo.reset()
+    cq = torch.compile(q, backend=backend, fullgraph=True)
+    with torch.no_grad():
+        want, eager, got = base(x), q(x), cq(x)
+        got2 = cq(x * 0.5)  # a second call reuses the graph
+        eager2 = q(x * 0.5)
+    assert got.dtype == dtype and got.shape == want.shape
+    assert _sqnr(f8, want, got) > 20
+    if backend != "inductor":
+        assert torch.equal(got, eager) and torch.equal(got2, eager2)
+    else:  # the compiler fuses SiLU and the product in fp32: last-bit differences in what the second linear sees
+        assert _sqnr(f8, eager, got) > 25 and _sqnr(f8, eager2, got2) > 25
+
+
 @pytest.mark.parametrize("shape,bias", [((3, 40, 512), True), ((130, 448), False), ((7, 200), True), ((64, 4096), True)])
 @pytest.mark.parametrize("static", [False, True])
 def test_fast_path_equals_the_composed_float8tensor_route_and_the_oracle(f8, shape, bias, static):
