@@ -254,8 +254,9 @@ def test_whole_delayed_scaling_step_as_one_graph(f8):
 
 
 @pytest.mark.parametrize("backend", ["eager", "aot_eager"])
-def test_delayed_scaling_and_inference_modules_run_outside_the_graph(f8, backend):
-    """State-carrying modules are not traced (graph break); compiled and eager runs still agree exactly."""
+def test_delayed_scaling_with_python_state_runs_outside_the_graph(f8, backend):
+    """Modules that keep Python state between calls (amax initialisation, pre/post-forward flags) are not traced (graph
+    break); compiled and eager runs still agree exactly.  The inference module, which keeps none, is checked as well."""
     from float8_experimental_amd.inference import ActivationCasting, QuantConfig, quantize_to_float8
 
     torch.manual_seed(2)
