@@ -21,6 +21,25 @@ namespace f8mi {
 #ifndef F8MI_CAST_REVERSE_WALK
 #define F8MI_CAST_REVERSE_WALK 0
 #endif
+#ifndef F8MI_CAST_NT_STORES   // measurement builds only: non-temporal stores of the fp8 bytes (16 % slower: 139 -> 161 us
+#define F8MI_CAST_NT_STORES 0  // per launch in the benchmark step, alternated three times on one box)
+#endif
+
+typedef uint32_t cast_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store8(uint8_t* p, uint32_t lo, uint32_t hi) {
+#if F8MI_CAST_NT_STORES
+    __builtin_nontemporal_store((cast_u32x2){lo, hi}, (cast_u32x2*)p);
+#else
+    *(uint2*)p = make_uint2(lo, hi);
+#endif
+}
+__device__ __forceinline__ void store16(uint8_t* p, uint4 v) {
+#if F8MI_CAST_NT_STORES
+    __builtin_nontemporal_store((u32x4){v.x, v.y, v.z, v.w}, (u32x4*)p);
+#else
+    *(uint4*)p = v;
+#endif
+}
 
 constexpr int CAST_THREADS = 256;
 constexpr int CAST_TILE = 128;
@@ -255,7 +274,7 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
                 // k-blocked: [cols/64][rows][64] (cols % 64 == 0, checked by the host)
                 uint8_t* p = out_kb ? out + ((col >> 6) * rows + row) * 64 + (col & 63) : out + row * cols + col;
                 if (out_vec) {  // cols % 8 == 0 implies col + 8 <= cols
-                    *(uint2*)p = make_uint2(lo[j], hi[j]);
+                    store8(p, lo[j], hi[j]);
                 } else {
 #pragma unroll
                     for (int i = 0; i < 8; i++)
@@ -289,7 +308,7 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
                 // k-blocked: [rows/64][cols][64] (rows % 64 == 0, checked by the host)
                 uint8_t* dst = out_t_kb ? out_t + ((gr >> 6) * cols + gc) * 64 + (gr & 63) : out_t + gc * rows + gr;
                 if (t_vec) {  // rows % 16 == 0 implies gr + 16 <= rows
-                    *(uint4*)dst = v;
+                    store16(dst, v);
                 } else {
                     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
