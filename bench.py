@@ -191,6 +191,42 @@ def probe_mfma(torch, random_data, iters=4000, operands=None):
     return out.value if rc == 0 else None
 
 
+def vendor_scaled_mm(torch, layers, m, flop_step, iters):
+    """The same twelve products through torch._scaled_mm (hipBLASLt), back to back, on row-major fp8 operands with the
+    transposed copies it needs made beforehand -- a reference point for the GEMM kernel, outside the timed region.
+    None where the installed torch refuses a product (format pair or layout)."""
+    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+    try:
+        one = torch.ones((), device="cuda:0")
+        ops = []
+        for name, k, n, lin, mod, x, dy in layers:
+            x8 = x.detach().clamp(-448, 448).to(E4)                         # [m, k]
+            w8 = (lin.weight.detach() * 64).clamp(-448, 448).to(E4)        # [n, k]
+            g8 = (dy * 1e4).clamp(-57344, 57344).to(E5)                     # [m, n]
+            w8t = w8.view(torch.uint8).t().contiguous().view(E4)           # [k, n]
+            g8t = g8.view(torch.uint8).t().contiguous().view(E5)           # [n, m]
+            x8t = x8.view(torch.uint8).t().contiguous().view(E4)           # [k, m]
+            # a row-major [rows, inner], b column-major [inner, cols] = .t() of a row-major [cols, inner]
+            ops.append(((x8, w8.t()), (g8, w8t.t()), (g8t, x8t.t())))
+
+        def run():
+            for trio in ops:
+                for a, b in trio:
+                    torch._scaled_mm(a, b, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+
+        run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            run()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / iters
+        return {"TFLOP/s": flop_step / dt / 1e12, "ms_per_12_gemms": dt * 1e3, "iterations": iters,
+                "what": "torch._scaled_mm (hipBLASLt), bf16 output, unit scales"}
+    except Exception as e:  # a product this torch build does not take
+        return {"TFLOP/s": None, "error": f"{type(e).__name__}: {str(e)[:160]}"}
+
+
 def cpu_baseline(torch, target_s):
     """The oracle's emulate=True restatement (fp32 dequant + torch.mm on the host) on token slices of the benchmark
     shapes, smallest weight first, until about ``target_s`` seconds of CPU work have been timed."""
@@ -316,7 +352,7 @@ def main():
 
     # ---- the twelve GEMMs of a step alone, back to back on operands cast beforehand (untimed for `value`): what the
     # matrix-core kernel sustains, and the socket power and shader clock it runs at, without the cast phases in between
-    gemm_loop = mfma_real = None
+    gemm_loop = mfma_real = vendor = None
     if args.scaling == "dynamic":
         E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
         ops = []
@@ -349,6 +385,7 @@ def main():
         # the same register-only loop on the fp8 bytes the benchmark's GEMMs actually multiply (x8 of the first shape)
         mfma_real = probe_mfma(torch, True, operands=ops[0][0])
         del ops
+        vendor = vendor_scaled_mm(torch, layers, m, flop_step, max(4, args.steps))
 
     # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
     mfma_zero = probe_mfma(torch, False)
@@ -390,6 +427,7 @@ def main():
             "mfma_only_benchmark_operands_TFLOP/s": mfma_real,
             "frac_of_mfma_only_random": gemm_tflops / mfma_random if mfma_random else None,
             "gemms_back_to_back": gemm_loop,
+            "vendor_scaled_mm_back_to_back": vendor,
         },
         "telemetry": telemetry,
         "hbm_kernels": hbm,
