@@ -168,10 +168,13 @@ def timed(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def probe_mfma(torch, random_data, iters=4000, operands=None):
-    """TFLOP/s of a register-only fp8 MFMA loop on every CU: the matrix cores' ceiling with no memory traffic, on zero
-    operands (clock limit), random ones (power limit) or -- ``operands``: an fp8 tensor of at least 256 KiB -- the bytes
-    of a real tensor.  From libf8mi_probe.so, a bench-only helper next to the library."""
+def probe_mfma(torch, random_data, iters=4000, operands=None, seconds=0.8):
+    """Register-only fp8 MFMA loop on every CU: what the matrix cores sustain with no memory traffic, on zero operands
+    (clock limit), random ones (the chip's power / current limits) or -- ``operands``: an fp8 tensor of at least
+    256 KiB -- the bytes of a real tensor.  The loop runs for ``seconds`` and the rate of the last third is reported,
+    with the socket power and shader clock over that third: the power management takes some hundred milliseconds to
+    settle, and a single 2 ms launch right after the GEMMs reads the clock they left, not the loop's own.
+    From libf8mi_probe.so, a bench-only helper next to the library."""
     import ctypes as C
 
     path = os.path.join(ROOT, "float8_experimental_amd", "libf8mi_probe.so")
@@ -186,45 +189,77 @@ def probe_mfma(torch, random_data, iters=4000, operands=None):
         scratch[:1 << 18].copy_(operands.reshape(-1).view(torch.uint8)[:1 << 18])
         mode = 2
     out = C.c_double(0.0)
-    rc = lib.f8mi_probe_mfma(mode, iters, scratch.data_ptr(), scratch.numel(), C.byref(out),
-                             torch.cuda.current_stream().cuda_stream)
-    return out.value if rc == 0 else None
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def once():
+        rc = lib.f8mi_probe_mfma(mode, iters, scratch.data_ptr(), scratch.numel(), C.byref(out), stream)
+        return out.value if rc == 0 else None
+
+    t_end = time.perf_counter() + seconds * 2.0 / 3.0
+    while time.perf_counter() < t_end:
+        if once() is None:
+            return None
+    tele = Telemetry()
+    tele.start()
+    vals = []
+    t_end = time.perf_counter() + seconds / 3.0
+    while time.perf_counter() < t_end:
+        vals.append(once())
+    t = tele.stop() or {}
+    return {"TFLOP/s": sum(vals) / len(vals), "socket_power_W": t.get("socket_power_W_mean"), "sclk_MHz": t.get("sclk_MHz_mean")}
 
 
-def vendor_scaled_mm(torch, layers, m, flop_step, iters):
-    """The same twelve products through torch._scaled_mm (hipBLASLt), back to back, on row-major fp8 operands with the
-    transposed copies it needs made beforehand -- a reference point for the GEMM kernel, outside the timed region.
-    None where the installed torch refuses a product (format pair or layout)."""
+def vendor_scaled_mm(torch, _native, layers, m, flop_step, iters):
+    """The same twelve products through torch._scaled_mm (hipBLASLt) on row-major fp8 operands with the transposed
+    copies it needs made beforehand -- a reference point for the GEMM kernel, outside the timed region: all twelve back
+    to back, and each product alone against this library's kernel on the same bytes (one fp8 copy per tensor, read as
+    it lies or transposed).  An "error" entry where the installed torch refuses a product (format pair or layout)."""
     E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
-    try:
-        one = torch.ones((), device="cuda:0")
-        ops = []
-        for name, k, n, lin, mod, x, dy in layers:
-            x8 = x.detach().clamp(-448, 448).to(E4)                         # [m, k]
-            w8 = (lin.weight.detach() * 64).clamp(-448, 448).to(E4)        # [n, k]
-            g8 = (dy * 1e4).clamp(-57344, 57344).to(E5)                     # [m, n]
-            w8t = w8.view(torch.uint8).t().contiguous().view(E4)           # [k, n]
-            g8t = g8.view(torch.uint8).t().contiguous().view(E5)           # [n, m]
-            x8t = x8.view(torch.uint8).t().contiguous().view(E4)           # [k, m]
-            # a row-major [rows, inner], b column-major [inner, cols] = .t() of a row-major [cols, inner]
-            ops.append(((x8, w8.t()), (g8, w8t.t()), (g8t, x8t.t())))
+    bf16 = torch.bfloat16
+    rowmajor = lambda t: t.permute(1, 0, 2).reshape(t.shape[1], -1).contiguous()
+    transposed = lambda t: t.view(torch.uint8).t().contiguous().view(t.dtype)
 
-        def run():
-            for trio in ops:
-                for a, b in trio:
-                    torch._scaled_mm(a, b, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
-
-        run()
+    def timed_loop(fn, n):
+        fn()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(iters):
-            run()
+        for _ in range(n):
+            fn()
         torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / iters
-        return {"TFLOP/s": flop_step / dt / 1e12, "ms_per_12_gemms": dt * 1e3, "iterations": iters,
-                "what": "torch._scaled_mm (hipBLASLt), bf16 output, unit scales"}
+        return (time.perf_counter() - t0) / n
+
+    try:
+        per_gemm, vendor_all, ours_all = [], [], []
+        for name, k, n, lin, mod, x, dy in layers:
+            x8, _, sx = _native.cast_dynamic(x.detach(), E4, out_kblock=True)
+            w8, _, sw = _native.cast_dynamic(lin.weight.detach(), E4, out_kblock=True)
+            g8, _, sg = _native.cast_dynamic(dy, E5, out_kblock=True)
+            x8r, w8r, g8r = rowmajor(x8), rowmajor(w8), rowmajor(g8)
+            w8t, g8t, x8t = transposed(w8r), transposed(g8r), transposed(x8r)
+            # torch._scaled_mm(a, b): a row-major [rows, inner], b column-major [inner, cols] = .t() of a row-major [cols, inner]
+            products = (
+                ("forward", lambda: _native.gemm_nt_kb(x8, sx, w8, sw, bf16),
+                 lambda: torch._scaled_mm(x8r, w8r.t(), scale_a=sx, scale_b=sw, out_dtype=bf16)),
+                ("grad_input", lambda: _native.gemm_kb_ex(g8, False, sg, w8, True, sw, bf16),
+                 lambda: torch._scaled_mm(g8r, w8t.t(), scale_a=sg, scale_b=sw, out_dtype=bf16)),
+                ("grad_weight", lambda: _native.gemm_kb_ex(g8, True, sg, x8, True, sx, bf16),
+                 lambda: torch._scaled_mm(g8t, x8t.t(), scale_a=sg, scale_b=sx, out_dtype=bf16)),
+            )
+            flop = 2.0 * m * k * n
+            for what, ours, theirs in products:
+                t_ours, t_theirs = timed_loop(ours, iters), timed_loop(theirs, iters)
+                per_gemm.append({"shape": name, "product": what, "this_library_TFLOP/s": flop / t_ours / 1e12,
+                                 "scaled_mm_TFLOP/s": flop / t_theirs / 1e12})
+                vendor_all.append(t_theirs)
+                ours_all.append(t_ours)
+            del x8, w8, g8, x8r, w8r, g8r, w8t, g8t, x8t, products
+        ours_ms = sum(ours_all) * 1e3
+        return {"what": "torch._scaled_mm (hipBLASLt), bf16 output; each product alone, back to back with itself",
+                "scaled_mm_TFLOP/s": flop_step / sum(vendor_all) / 1e12, "scaled_mm_ms_per_12_gemms": sum(vendor_all) * 1e3,
+                "this_library_TFLOP/s": flop_step / (ours_ms * 1e-3) / 1e12, "this_library_ms_per_12_gemms": ours_ms,
+                "per_gemm": per_gemm}
     except Exception as e:  # a product this torch build does not take
-        return {"TFLOP/s": None, "error": f"{type(e).__name__}: {str(e)[:160]}"}
+        return {"scaled_mm_TFLOP/s": None, "error": f"{type(e).__name__}: {str(e)[:160]}"}
 
 
 def cpu_baseline(torch, target_s):
@@ -385,7 +420,7 @@ def main():
         # the same register-only loop on the fp8 bytes the benchmark's GEMMs actually multiply (x8 of the first shape)
         mfma_real = probe_mfma(torch, True, operands=ops[0][0])
         del ops
-        vendor = vendor_scaled_mm(torch, layers, m, flop_step, max(4, args.steps))
+        vendor = vendor_scaled_mm(torch, _native, layers, m, flop_step, max(4, args.steps))
 
     # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
     mfma_zero = probe_mfma(torch, False)
@@ -422,12 +457,12 @@ def main():
             "launches": n_gemm,
             "avg_launch_ms": ms_gemm / max(n_gemm, 1),
             "flop_per_launch": flop_gemm / max(n_gemm, 1),
-            "mfma_only_zero_operands_TFLOP/s": mfma_zero,
-            "mfma_only_random_operands_TFLOP/s": mfma_random,
-            "mfma_only_benchmark_operands_TFLOP/s": mfma_real,
-            "frac_of_mfma_only_random": gemm_tflops / mfma_random if mfma_random else None,
+            "mfma_only_zero_operands": mfma_zero,
+            "mfma_only_random_operands": mfma_random,
+            "mfma_only_benchmark_operands": mfma_real,
+            "frac_of_mfma_only_random": gemm_tflops / mfma_random["TFLOP/s"] if mfma_random else None,
             "gemms_back_to_back": gemm_loop,
-            "vendor_scaled_mm_back_to_back": vendor,
+            "vendor_scaled_mm": vendor,
         },
         "telemetry": telemetry,
         "hbm_kernels": hbm,

@@ -12,6 +12,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #ifndef F8MI_WALK_GROUP
 #define F8MI_WALK_GROUP 4       // width of the bands the walk sweeps, in tiles
 #endif
+#ifndef F8MI_DMA_CACHE_POLICY   // cache-policy modifiers of the operand DMA (" nt", " sc1", ...), for measurement builds
+#define F8MI_DMA_CACHE_POLICY ""
+#endif
 #ifndef F8MI_WALK_XCD_CHUNK
 #define F8MI_WALK_XCD_CHUNK 0   // 0: each XCD owns one contiguous run of the tile order
 #endif
@@ -24,7 +27,7 @@ static_assert(DMA16_LDS >= EPI_BYTES, "the C staging tile reuses the slabs");
 
 __device__ __forceinline__ void dma16b(const uint8_t* base, uint32_t voff, uint32_t lds_addr) {
     // M0 carries the LDS address; one wait state between the scalar write of M0 and its use
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds_addr) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" F8MI_DMA_CACHE_POLICY ::"v"(voff), "s"(base), "s"(lds_addr) : "memory");
 }
 
 // acc += first (16 rows x 128 k, format F1) * second^T (16 rows x 128 k, format F2); formats 0 = e4m3, 1 = e5m2.
