@@ -18,6 +18,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #ifndef F8MI_WALK_XCD_CHUNK
 #define F8MI_WALK_XCD_CHUNK 0   // 0: each XCD owns one contiguous run of the tile order
 #endif
+#ifndef F8MI_WALK_SHORT_SIDE
+#define F8MI_WALK_SHORT_SIDE 0  // 1: sweep the bands along the shorter side of the tile grid
+#endif
 
 constexpr int SLAB_BYTES = 256 * 128;   // one operand, one step
 constexpr int HALF_BYTES = 256 * 64;    // one 64-deep unit of it
@@ -220,7 +223,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
     // 14.2 GB per launch / 2982 TFLOP/s, 2 tiles 7.8 / 3190, 4 tiles 5.2 / 3250, 8 tiles 5.2 / 3259, 16 tiles - / 3187.
     constexpr int GROUP = F8MI_WALK_GROUP;
     int tm, tn;
-    if (tiles_m > tiles_n) {
+    if ((tiles_m > tiles_n) != (F8MI_WALK_SHORT_SIDE != 0)) {
         const int width = GROUP * tiles_m;
         const int first_n = (lid / width) * GROUP;
         const int gsz = min(tiles_n - first_n, GROUP);
