@@ -168,10 +168,11 @@ def timed(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def probe_mfma(torch, random_data, iters=4000, operands=None, seconds=0.8):
+def probe_mfma(torch, random_data, iters=4000, operands=None, seconds=0.8, order=0, idle_w=None):
     """Register-only fp8 MFMA loop on every CU: what the matrix cores sustain with no memory traffic, on zero operands
     (clock limit), random ones (the chip's power / current limits) or -- ``operands``: an fp8 tensor of at least
-    256 KiB -- the bytes of a real tensor.  The loop runs for ``seconds`` and the rate of the last third is reported,
+    256 KiB -- the bytes of a real tensor.  ``order``: which operand changes from one instruction to the next (0 the
+    first, as in the GEMM; 1 the second; 2 both; 3 neither for eight in a row).  The loop runs for ``seconds`` and the rate of the last third is reported,
     with the socket power and shader clock over that third: the power management takes some hundred milliseconds to
     settle, and a single 2 ms launch right after the GEMMs reads the clock they left, not the loop's own.
     From libf8mi_probe.so, a bench-only helper next to the library."""
@@ -192,7 +193,7 @@ def probe_mfma(torch, random_data, iters=4000, operands=None, seconds=0.8):
     stream = torch.cuda.current_stream().cuda_stream
 
     def once():
-        rc = lib.f8mi_probe_mfma(mode, iters, scratch.data_ptr(), scratch.numel(), C.byref(out), stream)
+        rc = lib.f8mi_probe_mfma(mode + 16 * order, iters, scratch.data_ptr(), scratch.numel(), C.byref(out), stream)
         return out.value if rc == 0 else None
 
     t_end = time.perf_counter() + seconds * 2.0 / 3.0
@@ -206,7 +207,10 @@ def probe_mfma(torch, random_data, iters=4000, operands=None, seconds=0.8):
     while time.perf_counter() < t_end:
         vals.append(once())
     t = tele.stop() or {}
-    return {"TFLOP/s": sum(vals) / len(vals), "socket_power_W": t.get("socket_power_W_mean"), "sclk_MHz": t.get("sclk_MHz_mean")}
+    out = {"TFLOP/s": sum(vals) / len(vals), "socket_power_W": t.get("socket_power_W_mean"), "sclk_MHz": t.get("sclk_MHz_mean")}
+    if idle_w and out["socket_power_W"]:
+        out["pJ_per_flop_above_idle"] = (out["socket_power_W"] - idle_w) / out["TFLOP/s"]
+    return out
 
 
 def vendor_scaled_mm(torch, _native, layers, m, flop_step, iters):
@@ -325,6 +329,13 @@ def main():
         sync = lambda: f8.sync_float8_amax_and_scale_history(model)
     flop_per_shape = {name: 3 * 2.0 * m * k * n for name, k, n, *_ in layers}
     flop_step = sum(flop_per_shape.values())
+    # socket power with the tensors resident and nothing running, for the energy figures below
+    torch.cuda.synchronize()
+    time.sleep(0.5)
+    idle = Telemetry()
+    idle.start()
+    time.sleep(0.3)
+    idle_w = (idle.stop() or {}).get("socket_power_W_mean")
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -405,11 +416,12 @@ def main():
                     _native.gemm_kb_ex(g8, True, sg, x8, True, sx, torch.bfloat16)
 
         if all(_native.tn_ok(m, k, n) for _, k, n, *_ in layers):
-            gemms()
+            iters = max(8, 2 * args.steps)
+            for _ in range(iters):  # untimed: power and clock settle over some hundred milliseconds
+                gemms()
             torch.cuda.synchronize()
             tele = Telemetry()
             tele.start()
-            iters = max(8, 2 * args.steps)
             t0 = time.perf_counter()
             for _ in range(iters):
                 gemms()
@@ -417,14 +429,19 @@ def main():
             dt = (time.perf_counter() - t0) / iters
             gemm_loop = {"TFLOP/s": flop_step / dt / 1e12, "frac_of_fp8_peak": flop_step / dt / 1e12 / PEAK_FP8_TFLOPS,
                          "ms_per_12_gemms": dt * 1e3, "iterations": iters, "telemetry": tele.stop()}
+            if gemm_loop["telemetry"] and idle_w:
+                # joules per flop on top of what the idle socket draws: under the power cap this, not the number of
+                # stalled cycles, is what sets the rate
+                gemm_loop["idle_socket_power_W"] = idle_w
+                gemm_loop["pJ_per_flop_above_idle"] = (gemm_loop["telemetry"]["socket_power_W_mean"] - idle_w) / gemm_loop["TFLOP/s"]
         # the same register-only loop on the fp8 bytes the benchmark's GEMMs actually multiply (x8 of the first shape)
-        mfma_real = probe_mfma(torch, True, operands=ops[0][0])
+        mfma_real = probe_mfma(torch, True, operands=ops[0][0], idle_w=idle_w)
         del ops
         vendor = vendor_scaled_mm(torch, _native, layers, m, flop_step, max(4, args.steps))
 
     # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
-    mfma_zero = probe_mfma(torch, False)
-    mfma_random = probe_mfma(torch, True)
+    mfma_zero = probe_mfma(torch, False, idle_w=idle_w)
+    mfma_random = probe_mfma(torch, True, idle_w=idle_w)
 
     out = {
         "metric": "Float8Linear fwd+bwd TFLOP/s at LLaMa-2-70B shapes (1 GPU); cast GB/s",

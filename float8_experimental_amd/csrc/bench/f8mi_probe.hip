@@ -7,7 +7,9 @@
 //
 //   int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, size_t scratch_bytes, double* tflops, void* stream)
 //     random_data 0: all-zero operands, 1: random finite e4m3 bytes, 2: the first 256 KiB of scratch_dev as the
-//     caller left them (fp8 bytes of a real tensor);  scratch_dev: >= 1 MiB of device memory of the caller's;  *tflops receives the rate.  Returns 0, or -1 (bad argument) / -3 (a HIP call failed).
+//     caller left them (fp8 bytes of a real tensor); plus 16 * order, which operand of consecutive instructions
+//     changes: order 0 the first (as in the GEMM: the second stays for eight), 1 the second, 2 both, 3 neither;
+//     scratch_dev: >= 1 MiB of device memory of the caller's;  *tflops receives the rate.  Returns 0, or -1 (bad argument) / -3 (a HIP call failed).
 #include <vector>
 
 #include <hip/hip_runtime.h>
@@ -19,6 +21,7 @@ namespace f8mi {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+template <int ORDER>
 __global__ __launch_bounds__(256) void mfma_probe_kernel(const int* __restrict__ in, float* __restrict__ out, int iters) {
     v8i a[4], b[4];
 #pragma unroll
@@ -40,7 +43,8 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const int* __restrict__
         for (int i = 0; i < 8; i++)
 #pragma unroll
             for (int j = 0; j < 8; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j & 3], a[i & 3], acc[i][j], 0, 0, 0, 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    b[(ORDER == 1 || ORDER == 3 ? i : j) & 3], a[(ORDER == 1 ? j : ORDER == 2 ? i + j : i) & 3], acc[i][j], 0, 0, 0, 0, 0, 0);
     }
     float s = 0.f;
 #pragma unroll
@@ -67,6 +71,10 @@ extern "C" int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, si
     int dev = 0, n_cu = 0;
     if (check_hip(hipGetDevice(&dev), "hipGetDevice") || check_hip(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute")) return -3;
     const size_t need = 65536 * sizeof(int) + (size_t)n_cu * 256 * sizeof(float);
+    const int order = random_data >> 4;
+    random_data &= 15;
+    if (order < 0 || order > 3 || random_data > 2) { fprintf(stderr, "f8mi_probe_mfma: unknown mode\n"); return -1; }
+    auto kern = order == 0 ? mfma_probe_kernel<0> : order == 1 ? mfma_probe_kernel<1> : order == 2 ? mfma_probe_kernel<2> : mfma_probe_kernel<3>;
     if (!scratch_dev || scratch_bytes < need || !tflops || iters < 1) { fprintf(stderr, "f8mi_probe_mfma: needs %zu bytes of device scratch, a result pointer and iters >= 1\n", need); return -1; }
     int* in = (int*)scratch_dev;
     float* out = (float*)((char*)scratch_dev + 65536 * sizeof(int));
@@ -92,9 +100,9 @@ extern "C" int f8mi_probe_mfma(int random_data, int iters, void* scratch_dev, si
     hipEvent_t e0, e1;
     if ((rc = check_hip(hipEventCreate(&e0), "hipEventCreate"))) return rc;
     if ((rc = check_hip(hipEventCreate(&e1), "hipEventCreate"))) { (void)hipEventDestroy(e0); return rc; }
-    hipLaunchKernelGGL(mfma_probe_kernel, dim3(n_cu), dim3(256), 0, stream, in, out, iters / 8 + 1);  // warm-up
+    hipLaunchKernelGGL(kern, dim3(n_cu), dim3(256), 0, stream, in, out, iters / 8 + 1);  // warm-up
     (void)hipEventRecord(e0, stream);
-    hipLaunchKernelGGL(mfma_probe_kernel, dim3(n_cu), dim3(256), 0, stream, in, out, iters);
+    hipLaunchKernelGGL(kern, dim3(n_cu), dim3(256), 0, stream, in, out, iters);
     (void)hipEventRecord(e1, stream);
     rc = check_hip(hipEventSynchronize(e1), "hipEventSynchronize");
     float ms = 0.f;
