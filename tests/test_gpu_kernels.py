@@ -752,10 +752,14 @@ def test_sync_and_init_match_oracle(nat):
             a_d = torch.from_numpy(amax.copy()).to(DEV).reshape(n, 1)
             h_d = torch.from_numpy(hist.copy()).to(DEV)
             s_d = torch.zeros(n, 1, device=DEV)
-            table = nat.sync_table(((a_d[i], h_d[i], s_d[i], (torch.float8_e4m3fn, torch.float8_e5m2)[fmts[i]])
-                                    for i in range(n)), torch.device(DEV))
-            nat.sync(table, H, fp16, wb)
+            entries = [(a_d[i], h_d[i], s_d[i], (torch.float8_e4m3fn, torch.float8_e5m2)[fmts[i]]) for i in range(n)]
+            nat.sync(nat.sync_table(entries, torch.device(DEV)), H, fp16, wb)
             got_s, got_h = s_d.cpu().numpy().reshape(-1), h_d.cpu().numpy()
+            # the same through the entry point that takes the entries as kernel arguments (32 per launch: 999 = 31 * 32 + 7)
+            h2_d = torch.from_numpy(hist.copy()).to(DEV)
+            s2_d = torch.zeros(n, 1, device=DEV)
+            nat.sync_host([(a_d[i], h2_d[i], s2_d[i], e[3]) for i, e in enumerate(entries)], H, fp16, wb)
+            assert torch.equal(s2_d.view(torch.int32), s_d.view(torch.int32)) and torch.equal(h2_d.view(torch.int32), h_d.view(torch.int32))
             for i in range(n):
                 h = hist[i].copy()
                 want = co.sync_entry(amax[i], h, int(fmts[i]), fp16, wb)
