@@ -60,3 +60,30 @@ def test_accumulator_reads_keep_their_distance_from_the_mfma_that_writes_them(li
                     f"{unit}:{i + 1}: {line.strip()} only {n_mfma - at_mfma} MFMAs and {nops} wait states after its MFMA")
         assert n_mfma > 0 and n_reads == 256, (unit, n_mfma, n_reads)  # 64 accumulator tiles of 4 registers, each read once
         start = end + 1
+
+
+@pytest.mark.parametrize("unit", UNITS)
+def test_every_lds_dma_sets_m0_itself_with_the_wait_state_it_needs(listings, unit):
+    """A global load into the LDS takes its LDS address from M0.  The scalar write of M0 needs one wait state before
+    the vector memory instruction that reads it, and nothing may change M0 in between: every such load must come
+    straight after `s_mov_b32 m0, ...` and `s_nop`, as the kernel's hand-written sequence has it."""
+    lines = [l.strip() for l in listings[unit]]
+    code = [l for l in lines if l and not l.startswith((";", ".", "//")) and not l.endswith(":")]
+    n = 0
+    for i, l in enumerate(code):
+        if l.startswith("global_load_lds_"):
+            n += 1
+            assert code[i - 1].startswith("s_nop"), f"{unit}: `{l}` follows `{code[i - 1]}`"
+            assert code[i - 2].startswith("s_mov_b32 m0,"), f"{unit}: `{l}`: M0 written by `{code[i - 2]}`"
+    assert n >= 12 * 16 * 3  # every instantiation has the prologue's 32 and at least two steps with 16
+
+
+@pytest.mark.parametrize("unit", UNITS)
+def test_no_spills_and_accumulators_stay_in_place(listings, unit):
+    """The kernel's register budget is exact (256 accumulator registers + the fragments of two steps): a build that
+    spills or moves accumulators through vector registers is a build that lost its schedule."""
+    text = "\n".join(listings[unit])
+    assert "scratch_store" not in text and "scratch_load" not in text
+    assert "v_accvgpr_mov" not in text
+    sizes = [int(x) for x in re.findall(r"; ScratchSize: (\d+)", text)]
+    assert sizes and not any(sizes)
