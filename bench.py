@@ -126,6 +126,9 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-bf16", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the oracle sample")
+    p.add_argument("--mfma-order", type=int, default=0, choices=[0, 1, 2, 3],
+                   help="register-only MFMA loop: which operand changes between consecutive instructions "
+                        "(0 the first, as in the GEMM; 1 the second; 2 both; 3 neither for eight in a row)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run one plain 1 GiB device-to-device copy (for scaling hardware byte counters of a profiler run)")
     return p.parse_args()
@@ -435,13 +438,13 @@ def main():
                 gemm_loop["idle_socket_power_W"] = idle_w
                 gemm_loop["pJ_per_flop_above_idle"] = (gemm_loop["telemetry"]["socket_power_W_mean"] - idle_w) / gemm_loop["TFLOP/s"]
         # the same register-only loop on the fp8 bytes the benchmark's GEMMs actually multiply (x8 of the first shape)
-        mfma_real = probe_mfma(torch, True, operands=ops[0][0], idle_w=idle_w)
+        mfma_real = probe_mfma(torch, True, operands=ops[0][0], idle_w=idle_w, order=args.mfma_order)
         del ops
         vendor = vendor_scaled_mm(torch, _native, layers, m, flop_step, max(4, args.steps))
 
     # the matrix cores' own ceiling on this box: register-only MFMA loop, clock-limited (zeros) and power-limited (random bytes)
-    mfma_zero = probe_mfma(torch, False, idle_w=idle_w)
-    mfma_random = probe_mfma(torch, True, idle_w=idle_w)
+    mfma_zero = probe_mfma(torch, False, idle_w=idle_w, order=args.mfma_order)
+    mfma_random = probe_mfma(torch, True, idle_w=idle_w, order=args.mfma_order)
 
     out = {
         "metric": "Float8Linear fwd+bwd TFLOP/s at LLaMa-2-70B shapes (1 GPU); cast GB/s",
