@@ -77,9 +77,12 @@ def _(a, a_scale, bt, b_scale, out_dtype, bias):
 # ---- the fused linear ----------------------------------------------------------------------------------------
 
 
-def _layout(t_rows: int, t_cols: int, kblock: bool):
-    """Shape of an fp8 operand with ``t_rows`` rows contracting over ``t_cols``."""
-    return (t_cols // _KB, t_rows, _KB) if kblock else (t_rows, t_cols)
+def _layout(t_rows: int, t_cols: int, layout: int):
+    """Shape of an fp8 operand with ``t_rows`` rows contracting over ``t_cols`` in layout ``_native.ROWMAJOR / KBLOCK /
+    KBLOCK_PAD``."""
+    if layout == _native.ROWMAJOR:
+        return (t_rows, t_cols)
+    return ((t_cols if layout == _native.KBLOCK else _native.padded_k(t_cols)) // _KB, t_rows, _KB)
 
 
 def _cast(t2d, float8_dtype, scale_buf, want_row, want_t, row_kb, t_kb):
@@ -124,7 +127,7 @@ def _linear_fwd_impl(x2, weight, need_dx, need_dw, scale_x, scale_w):
         x8, _, sx, ax = _cast(x2, e4m3_dtype, scale_x, True, False, True, False)
         w8, _, sw, aw = _cast(weight, e4m3_dtype, scale_w, True, False, True, False)
         return _native.gemm_nt_kb(x8, sx, w8, sw, x2.dtype), x8, w8, out_s(sx, scale_x), out_s(sw, scale_w), ax, aw
-    kb_fwd, kb_dx, kb_dw = _native.kblock_ok(k), _native.kblock_ok(n), _native.kblock_ok(m)
+    kb_fwd, kb_dx, kb_dw = _native.kblock_layout(k), _native.kblock_layout(n), _native.kblock_layout(m)
     x8, x8t, sx, ax = _cast(x2, e4m3_dtype, scale_x, True, need_dw, kb_fwd, kb_dw)
     w8, w8t, sw, aw = _cast(weight, e4m3_dtype, scale_w, True, need_dx, kb_fwd, kb_dx)
     y = _gemm(x8, sx, w8, sw, x2.dtype, kb_fwd)
@@ -142,7 +145,7 @@ def _(x2, weight, need_dx, need_dw, scale_x, scale_w):
     y = torch.empty((m, n), dtype=x2.dtype, device=x2.device)
     if _native.tn_ok(m, k, n):
         return y, f8((k // _KB, m, _KB)), f8((k // _KB, n, _KB)), s(scale_x), s(scale_w), a(scale_x), a(scale_w)
-    kb_dx, kb_dw = _native.kblock_ok(n), _native.kblock_ok(m)
+    kb_dx, kb_dw = _native.kblock_layout(n), _native.kblock_layout(m)
     return (y, f8(_layout(k, m, kb_dw)) if need_dw else f8((0,)), f8(_layout(k, n, kb_dx)) if need_dx else f8((0,)),
             s(scale_x), s(scale_w), a(scale_x), a(scale_w))
 
@@ -165,7 +168,7 @@ def _linear_bwd_impl(dy2, xs, ws, sx, sw, k, need_dx, need_dw, scale_g):
         dx = _native.gemm_kb_ex(g8, False, sg, ws, True, sw, dy2.dtype) if need_dx else empty()
         dw = _native.gemm_kb_ex(g8, True, sg, xs, True, sx, dy2.dtype) if need_dw else empty()
         return dx, dw, ag
-    kb_dx, kb_dw = _native.kblock_ok(n), _native.kblock_ok(m)
+    kb_dx, kb_dw = _native.kblock_layout(n), _native.kblock_layout(m)
     g8, g8t, sg, ag = _cast(dy2, e5m2_dtype, scale_g, need_dx, need_dw, kb_dx, kb_dw)
     dx = _gemm(g8, sg, ws, sw, dy2.dtype, kb_dx) if need_dx else empty()
     dw = _gemm(g8t, sg, xs, sx, dy2.dtype, kb_dw) if need_dw else empty()

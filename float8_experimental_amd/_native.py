@@ -13,7 +13,9 @@ from typing import Optional, Tuple
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# F8MI_LIB names another build of the library (same ABI) to load instead of the in-tree one
+# F8MI_LIB names another build of the library (same ABI) to load instead of the in-tree one: a switch for measurements
+# (tile walks, cache policies).  Such a build says so through f8mi_build_knobs() and is refused unless
+# F8MI_ALLOW_MEASUREMENT_BUILD=1 is set as well.
 LIB_PATH = os.environ.get("F8MI_LIB") or os.path.join(_HERE, "libf8mi.so")
 
 BF16, FP16, FP32 = 0, 1, 2
@@ -26,6 +28,8 @@ _F8 = {torch.float8_e4m3fn: E4M3FN, torch.float8_e5m2: E5M2}
 EXPORTS = (
     "f8mi_version",
     "f8mi_last_error",
+    "f8mi_build_knobs",
+    "f8mi_padded_k",
     "f8mi_device_info",
     "f8mi_workspace_bytes",
     "f8mi_gemm_nt_ws",
@@ -76,6 +80,10 @@ def lib() -> C.CDLL:
         L.f8mi_version.argtypes = []
         L.f8mi_last_error.restype = C.c_char_p
         L.f8mi_last_error.argtypes = []
+        L.f8mi_build_knobs.restype = C.c_char_p
+        L.f8mi_build_knobs.argtypes = []
+        L.f8mi_padded_k.restype = i64
+        L.f8mi_padded_k.argtypes = [i64]
         L.f8mi_device_info.restype = i32
         L.f8mi_device_info.argtypes = [i32, C.POINTER(i32), C.POINTER(i32), C.c_char_p, i32]
         L.f8mi_workspace_bytes.restype = C.c_size_t
@@ -118,8 +126,18 @@ def lib() -> C.CDLL:
         L.f8mi_prof_reset.argtypes = []
         L.f8mi_prof_read.restype = i32
         L.f8mi_prof_read.argtypes = [i32, C.POINTER(C.c_uint64), C.POINTER(C.c_double), C.POINTER(C.c_double)]
+        knobs = L.f8mi_build_knobs().decode()
+        if knobs and os.environ.get("F8MI_ALLOW_MEASUREMENT_BUILD") != "1":
+            raise Float8NativeError(
+                f"{LIB_PATH} is a measurement build ({knobs}), not the library as shipped; set "
+                "F8MI_ALLOW_MEASUREMENT_BUILD=1 to load it anyway")
         _lib = L
     return _lib
+
+
+def build_knobs() -> str:
+    """Measurement knobs the loaded library was compiled with ("" for the shipped build).  See f8mi_build_knobs."""
+    return lib().f8mi_build_knobs().decode()
 
 
 def _check(rc: int, what: str) -> None:
@@ -321,6 +339,43 @@ def amax_scale_multi(tensors, float8_dtype: torch.dtype, math_dtype: Optional[to
 
 KB = 64          # depth of one block of the k-blocked operand layout
 KB_MIN_K = 384   # shortest contraction the k-blocked GEMM takes
+ROWMAJOR, KBLOCK, KBLOCK_PAD = 0, 1, 2  # F8MI_LAYOUT_ROWMAJOR / _KBLOCK64 / _KBLOCK64_PAD128
+
+
+def padded_k(k: int) -> int:
+    """Contraction length of a zero-padded k-blocked operand: k rounded up to a multiple of 128 (f8mi_padded_k)."""
+    return -(-k // 128) * 128 if k > 0 else 0
+
+
+def kblock_layout(k: int) -> int:
+    """Layout code of the fp8 copies that a GEMM contracting over k reads fastest: k-blocked as it is when k is a
+    multiple of 64 (and at least 384), k-blocked with the contraction zero-padded to a multiple of 128 for any other k
+    that reaches 384 that way (a ragged layer: zeros add nothing to the product, which is the reference's own argument
+    for pad_tensor_for_matmul, float8_utils.py:206-247), row-major for a short contraction."""
+    if k % KB == 0 and k >= KB_MIN_K:
+        return KBLOCK
+    return KBLOCK_PAD if padded_k(k) >= KB_MIN_K else ROWMAJOR
+
+
+def linear_route(m: int, k: int, n: int):
+    """How the fused Float8Linear computes a layer of m tokens, k in_features, n out_features (needs no GPU):
+    {"one_copy": bool, product: (operand layout code, contraction length the GEMM runs over, kernel plan)} for the
+    products "output" (m x n over k), "grad_input" (m x k over n) and "grad_weight" (n x k over m)."""
+    route = {"one_copy": tn_ok(m, k, n)}
+    for name, (rows, cols, kc) in (("output", (m, n, k)), ("grad_input", (m, k, n)), ("grad_weight", (n, k, m))):
+        layout = KBLOCK if route["one_copy"] else kblock_layout(kc)
+        kc_run = padded_k(kc) if layout == KBLOCK_PAD else kc
+        route[name] = (layout, kc_run, gemm_plan(rows, cols, kc_run, aligned=layout != ROWMAJOR or kc % 16 == 0))
+    return route
+
+
+def _kb_alloc(rows: int, kc: int, layout: int, float8_dtype, device) -> torch.Tensor:
+    """Uninitialised k-blocked operand of ``rows`` rows contracting over ``kc``: [kc/64, rows, 64], kc padded for KBLOCK_PAD."""
+    if layout == KBLOCK:
+        assert kc % KB == 0, f"a k-blocked copy needs a contraction length that is a multiple of {KB}, got {kc} (use KBLOCK_PAD)"
+    else:
+        kc = padded_k(kc)
+    return torch.empty((kc // KB, rows, KB), dtype=float8_dtype, device=device)
 
 
 def tn_ok(m: int, k: int, n: int) -> bool:
@@ -341,14 +396,16 @@ def kblock_ok(k: int) -> bool:
 
 def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, product_dtype: Optional[torch.dtype] = None,
          want_out: bool = True, want_out_t: bool = False, amax_out: Optional[torch.Tensor] = None,
-         out_kblock: bool = False, out_t_kblock: bool = False):
+         out_kblock: int = 0, out_t_kblock: int = 0):
     """Saturated fp8 cast of a tensor viewed as [rows, cols=last dim].
 
     Returns (out, out_t): ``out`` has x's shape; ``out_t`` is the dense [cols, rows]
     transpose of the flattened 2-D view.  ``amax_out`` (fp32, 1 element), if given,
     receives max|x| computed in the same pass.  With ``out_kblock`` / ``out_t_kblock``
     the respective output is k-blocked instead: shape [cols/64, rows, 64] for ``out``
-    (``out[b, r, j] == rowmajor[r, 64*b + j]``), [rows/64, cols, 64] for ``out_t``.
+    (``out[b, r, j] == rowmajor[r, 64*b + j]``), [rows/64, cols, 64] for ``out_t``; the value
+    ``KBLOCK_PAD`` (2) instead of True pads the contraction with zero bytes to a multiple of 128 first
+    (any shape: [padded_k(cols)/64, rows, 64] and [padded_k(rows)/64, cols, 64]).
     See f8mi_cast / f8mi_cast_layout.
     """
     _require_gpu(x, "x")
@@ -358,17 +415,9 @@ def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, produc
         product_dtype = x.dtype
     out = out_t = None
     if want_out:
-        if out_kblock:
-            assert cols % KB == 0, f"k-blocked out needs cols % {KB} == 0, got {cols}"
-            out = torch.empty((cols // KB, rows, KB), dtype=float8_dtype, device=x.device)
-        else:
-            out = torch.empty(x.shape, dtype=float8_dtype, device=x.device)
+        out = _kb_alloc(rows, cols, int(out_kblock), float8_dtype, x.device) if out_kblock else torch.empty(x.shape, dtype=float8_dtype, device=x.device)
     if want_out_t:
-        if out_t_kblock:
-            assert rows % KB == 0, f"k-blocked out_t needs rows % {KB} == 0, got {rows}"
-            out_t = torch.empty((rows // KB, cols, KB), dtype=float8_dtype, device=x.device)
-        else:
-            out_t = torch.empty((cols, rows), dtype=float8_dtype, device=x.device)
+        out_t = _kb_alloc(cols, rows, int(out_t_kblock), float8_dtype, x.device) if out_t_kblock else torch.empty((cols, rows), dtype=float8_dtype, device=x.device)
     if amax_out is not None:
         assert amax_out.dtype == torch.float32 and amax_out.numel() == 1 and amax_out.device == x.device
     _check_device(x.device)
@@ -385,7 +434,7 @@ def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, produc
 
 
 def cast_dynamic(x: torch.Tensor, float8_dtype: torch.dtype, want_out: bool = True, want_out_t: bool = False,
-                 out_kblock: bool = False, out_t_kblock: bool = False):
+                 out_kblock: int = 0, out_t_kblock: int = 0):
     """(out, out_t, scale): ``amax_scale`` in x's dtype followed by ``cast`` with that scale, as one library call
     (hp_tensor_to_float8_dynamic of the reference); small tensors take a single launch.  See f8mi_cast_dynamic."""
     _require_gpu(x, "x")
@@ -393,17 +442,9 @@ def cast_dynamic(x: torch.Tensor, float8_dtype: torch.dtype, want_out: bool = Tr
     scale = torch.empty((), dtype=torch.float32, device=x.device)
     out = out_t = None
     if want_out:
-        if out_kblock:
-            assert cols % KB == 0, f"k-blocked out needs cols % {KB} == 0, got {cols}"
-            out = torch.empty((cols // KB, rows, KB), dtype=float8_dtype, device=x.device)
-        else:
-            out = torch.empty(x.shape, dtype=float8_dtype, device=x.device)
+        out = _kb_alloc(rows, cols, int(out_kblock), float8_dtype, x.device) if out_kblock else torch.empty(x.shape, dtype=float8_dtype, device=x.device)
     if want_out_t:
-        if out_t_kblock:
-            assert rows % KB == 0, f"k-blocked out_t needs rows % {KB} == 0, got {rows}"
-            out_t = torch.empty((rows // KB, cols, KB), dtype=float8_dtype, device=x.device)
-        else:
-            out_t = torch.empty((cols, rows), dtype=float8_dtype, device=x.device)
+        out_t = _kb_alloc(cols, rows, int(out_t_kblock), float8_dtype, x.device) if out_t_kblock else torch.empty((cols, rows), dtype=float8_dtype, device=x.device)
     ws = workspace(x.device)
     empty = rows * cols == 0  # torch hands out null pointers for empty tensors: only the scale is computed
     rc = lib().f8mi_cast_dynamic(xs.data_ptr() if not empty else None, rows, cols, ld, _DT[x.dtype], _F8[float8_dtype],
@@ -415,7 +456,7 @@ def cast_dynamic(x: torch.Tensor, float8_dtype: torch.dtype, want_out: bool = Tr
 
 
 def cast_dynamic_static(x: torch.Tensor, scale_out: torch.Tensor, out: Optional[torch.Tensor] = None,
-                        out_t: Optional[torch.Tensor] = None, out_kblock: bool = False, out_t_kblock: bool = False) -> None:
+                        out_t: Optional[torch.Tensor] = None, out_kblock: int = 0, out_t_kblock: int = 0) -> None:
     """``cast_dynamic`` into tensors the caller already holds, through the library's own static scratch: this
     function and the library call behind it allocate nothing (see f8mi_cast_dynamic_static).  ``x`` must be a 2-D
     view with unit column stride; ``out`` / ``out_t`` are fp8 tensors of rows*cols elements, ``scale_out`` one fp32

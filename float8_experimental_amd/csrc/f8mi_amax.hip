@@ -15,18 +15,7 @@ namespace f8mi {
 constexpr int AMAX_THREADS = 256;
 constexpr int AMAX_UNROLL = 8;  // 16-byte loads in flight per thread
 
-// Loads are non-temporal.  Measurement builds can read tensors of up to F8MI_AMAX_PLAIN_LOADS_MAX_BYTES with ordinary
-// loads instead (-DF8MI_AMAX_PLAIN_LOADS_MAX_BYTES=...), which leave the tensor in the 256 MB memory-side cache for
-// the cast that follows.  Measured in the benchmark step (kernel times from a trace, amax + cast of one tensor):
-//   every tensor with ordinary loads: 134 MB 59.7 -> 55.7 us, 168 MB 72.5 -> 71.6, but 268 MB 111.6 -> 121.4,
-//     470 MB 199.5 -> 238.4, 1.9 GB 774 -> 816 (the cast gains 3 - 10 %, the amax pass loses 30 - 70 %);
-//   only tensors up to 192 MB with ordinary loads: 134 MB 59.7 -> 66.9 us, 168 MB 72.5 -> 80.9 -- worse than either.
-// A line allocated in that cache pushes out a line that is there, and when that is a dirty line -- the fp8 copy or the
-// GEMM output written just before -- its write-back competes with the reads: what ordinary loads cost depends on what
-// the kernels before left in the cache, not on the tensor's size, and no size rule survives a change of neighbours.
-#ifndef F8MI_AMAX_PLAIN_LOADS_MAX_BYTES
-#define F8MI_AMAX_PLAIN_LOADS_MAX_BYTES 0
-#endif
+// Loads are non-temporal (F8MI_AMAX_PLAIN_LOADS_MAX_BYTES in f8mi_knobs.h has what ordinary loads were measured to cost).
 template <bool NT>
 __device__ __forceinline__ uint4 amax_load16(const uint4* p) {
     if constexpr (NT) return load_nt16(p);

@@ -80,6 +80,29 @@ extern "C" int f8mi_version(void) { return F8MI_VERSION; }
 
 extern "C" const char* f8mi_last_error(void) { return g_err; }
 
+extern "C" int64_t f8mi_padded_k(int64_t k) { return k <= 0 ? 0 : (k + 127) / 128 * 128; }
+
+// Names every measurement knob (f8mi_knobs.h) this build was compiled with a non-default value of; "" for the
+// shipped configuration.
+extern "C" const char* f8mi_build_knobs(void) {
+    static char knobs[256];
+    static std::once_flag once;
+    std::call_once(once, [] {
+        size_t n = 0;
+        auto add = [&](const char* name, long long value, long long dflt) {
+            if (value != dflt && n < sizeof(knobs)) n += (size_t)snprintf(knobs + n, sizeof(knobs) - n, "%s%s=%lld", n ? " " : "", name, value);
+        };
+        add("F8MI_WALK_GROUP", F8MI_WALK_GROUP, 4);
+        add("F8MI_WALK_XCD_CHUNK", F8MI_WALK_XCD_CHUNK, 0);
+        add("F8MI_WALK_SHORT_SIDE", F8MI_WALK_SHORT_SIDE, 0);
+        add("F8MI_DMA_CACHE_POLICY_SET", !F8MI_DMA_CACHE_POLICY_IS_DEFAULT, 0);
+        add("F8MI_CAST_REVERSE_WALK", F8MI_CAST_REVERSE_WALK, 0);
+        add("F8MI_CAST_NT_STORES", F8MI_CAST_NT_STORES, 0);
+        add("F8MI_AMAX_PLAIN_LOADS_MAX_BYTES", F8MI_AMAX_PLAIN_LOADS_MAX_BYTES, 0);
+    });
+    return knobs;
+}
+
 extern "C" size_t f8mi_workspace_bytes(void) { return WS_WORDS * sizeof(uint32_t); }
 
 extern "C" int f8mi_device_info(int device, int* cu_count, int* lds_bytes, char* arch, int arch_len) {

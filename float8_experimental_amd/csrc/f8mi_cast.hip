@@ -18,32 +18,22 @@
 
 namespace f8mi {
 
-#ifndef F8MI_CAST_REVERSE_WALK
-#define F8MI_CAST_REVERSE_WALK 0
-#endif
-#ifndef F8MI_CAST_NT_STORES   // measurement builds only: non-temporal stores of the fp8 bytes (16 % slower: 139 -> 161 us
-#define F8MI_CAST_NT_STORES 0  // per launch in the benchmark step, alternated three times on one box)
-#endif
-
-typedef uint32_t cast_u32x2 __attribute__((ext_vector_type(2)));
+// The fp8 bytes leave as 8-byte (row-major copy) and 16-byte (transposed copy) stores at whatever alignment the
+// output's row pitch gives them.
 __device__ __forceinline__ void store8(uint8_t* p, uint32_t lo, uint32_t hi) {
 #if F8MI_CAST_NT_STORES
-    __builtin_nontemporal_store((cast_u32x2){lo, hi}, (cast_u32x2*)p);
+    __builtin_nontemporal_store((u32x2){lo, hi}, (u32x2_any*)p);
 #else
-    *(uint2*)p = make_uint2(lo, hi);
+    store8_any(p, lo, hi);
 #endif
 }
 __device__ __forceinline__ void store16(uint8_t* p, uint4 v) {
 #if F8MI_CAST_NT_STORES
-    __builtin_nontemporal_store((u32x4){v.x, v.y, v.z, v.w}, (u32x4*)p);
+    __builtin_nontemporal_store((u32x4){v.x, v.y, v.z, v.w}, (u32x4_any*)p);
 #else
-    *(uint4*)p = v;
+    store16_any(p, v);
 #endif
 }
-
-#ifndef F8MI_CAST_NO_CLAMP   // measurement builds only (wrong beyond the fp8 range): without the clamp's six vector instructions
-#define F8MI_CAST_NO_CLAMP 0  // per element pair (of fourteen) the kernel is 0.5 % faster (139.5 -> 138.8 us per launch in the
-#endif                        // benchmark step, alternated twice on one box): the arithmetic is not what bounds it
 
 constexpr int CAST_THREADS = 256;
 constexpr int CAST_TILE = 128;
@@ -81,13 +71,8 @@ __device__ __forceinline__ void scale_clamp2(float x0, float x1, float scale, fl
         p0 = round_to_fp16(p0);
         p1 = round_to_fp16(p1);
     }
-#if F8MI_CAST_NO_CLAMP
-    y0 = p0;
-    y1 = p1;
-#else
     y0 = clamp_keep_nan(p0, fmax);
     y1 = clamp_keep_nan(p1, fmax);
-#endif
 }
 
 // 4 dwords (rows 0..3, 4 bytes each = columns 0..3) -> 4 dwords (column c: rows 0..3)
@@ -138,8 +123,10 @@ __device__ __forceinline__ uint32_t absmax_done(uint32_t m) {
     else return fold16(m);
 }
 
-// Loads 8 elements of row `row` starting at column `col`; out-of-range elements read as +0.
-template <int DT, bool VEC>
+// Loads 8 elements of row `row` starting at column `col`; out-of-range elements read as +0.  Eight elements inside the
+// row are one 16-byte load (two for fp32) whatever the row pitch: a row only has to start at a multiple of the
+// element size.
+template <int DT>
 __device__ __forceinline__ void load_row8(Row8<DT>& r, const void* x, int64_t row, int64_t col, int64_t rows,
                                           int64_t cols, int64_t ld) {
     constexpr int ESZ = DT == F8MI_FP32 ? 4 : 2;
@@ -148,12 +135,11 @@ __device__ __forceinline__ void load_row8(Row8<DT>& r, const void* x, int64_t ro
     for (int i = 0; i < NW; i++) r.w[i] = 0u;
     if (row >= rows || col >= cols) return;
     const char* p = (const char*)x + (row * ld + col) * ESZ;
-    if (VEC && col + 8 <= cols) {
-        const uint4* pv = (const uint4*)p;
-        uint4 v0 = load_nt16(pv);
+    if (col + 8 <= cols) {
+        uint4 v0 = load_nt16_any(p);
         r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v0.z; r.w[3] = v0.w;
         if constexpr (DT == F8MI_FP32) {
-            uint4 v1 = load_nt16(pv + 1);
+            uint4 v1 = load_nt16_any(p + 16);
             r.w[4] = v1.x; r.w[5] = v1.y; r.w[6] = v1.z; r.w[7] = v1.w;
         }
     } else {
@@ -167,7 +153,8 @@ __device__ __forceinline__ void load_row8(Row8<DT>& r, const void* x, int64_t ro
     }
 }
 
-template <int DT, int PROD, int FMT, bool VEC>
+// out_kb / out_t_kb: F8MI_LAYOUT_* code of the respective output.
+template <int DT, int PROD, int FMT>
 __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
                                                             int64_t ld, const float* __restrict__ scale_dev,
                                                             uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
@@ -227,7 +214,7 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
 #pragma unroll
     for (int h = 0; h < 2; h++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) load_row8<DT, VEC>(in[h][j], x, r0 + 64 * h + 4 * b + j, col, rows, cols, ld);
+        for (int j = 0; j < 4; j++) load_row8<DT>(in[h][j], x, r0 + 64 * h + 4 * b + j, col, rows, cols, ld);
 
     // The scale: given -- or, for dynamic scaling, derived here from the per-workgroup maxima the amax kernel left in
     // amax_ws (every wave of every workgroup reduces the <= 1024 words itself; saves the one-block launch that would do
@@ -266,7 +253,16 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
         m = absmax_done<DT>(m);
     }
 
-    const bool out_vec = (cols % 8 == 0) && ((uintptr_t)out % 8 == 0);
+    // Zero-padded k-blocked outputs (F8MI_LAYOUT_KBLOCK64_PAD128): the tile grid ends exactly where the padding does, so
+    // a tile writes all of its 128 columns (`out`) or rows (`out_t`); what lies past the tensor's edge is forced to
+    // zero bytes (elements read as +0 would become NaN codes under a NaN scale).
+    const bool pad = out_kb == F8MI_LAYOUT_KBLOCK64_PAD128 || out_t_kb == F8MI_LAYOUT_KBLOCK64_PAD128;
+    uint32_t keep_lo = 0xffffffffu, keep_hi = 0xffffffffu;  // bytes of the lane's eight columns that lie inside the row
+    if (pad && col + 8 > cols) {
+        const int valid = col < cols ? (int)(cols - col) : 0;
+        keep_lo = valid >= 4 ? 0xffffffffu : (valid ? (1u << (8 * valid)) - 1u : 0u);
+        keep_hi = valid > 4 ? (1u << (8 * (valid - 4))) - 1u : 0u;
+    }
 #pragma unroll
     for (int h = 0; h < 2; h++) {
         uint32_t lo[4], hi[4];
@@ -279,10 +275,14 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
             lo[j] = cvt4_fp8<FMT>(f[0], f[1], f[2], f[3]);
             hi[j] = cvt4_fp8<FMT>(f[4], f[5], f[6], f[7]);
             const int64_t row = r0 + 64 * h + 4 * b + j;
-            if (out && row < rows && col < cols) {
-                // k-blocked: [cols/64][rows][64] (cols % 64 == 0, checked by the host)
+            if (pad) {
+                lo[j] = row < rows ? lo[j] & keep_lo : 0u;
+                hi[j] = row < rows ? hi[j] & keep_hi : 0u;
+            }
+            if (out && row < rows && (col < cols || out_kb == F8MI_LAYOUT_KBLOCK64_PAD128)) {
+                // k-blocked: [cols/64][rows][64] (cols % 64 == 0 or padded to it: the eight columns are always whole)
                 uint8_t* p = out_kb ? out + ((col >> 6) * rows + row) * 64 + (col & 63) : out + row * cols + col;
-                if (out_vec) {  // cols % 8 == 0 implies col + 8 <= cols
+                if (out_kb || col + 8 <= cols) {
                     store8(p, lo[j], hi[j]);
                 } else {
 #pragma unroll
@@ -304,7 +304,6 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
 
     if (out_t) {
         __syncthreads();
-        const bool t_vec = (rows % 16 == 0) && ((uintptr_t)out_t % 16 == 0);
 #pragma unroll
         for (int p = 0; p < 4; p++) {
             const int id = p * CAST_THREADS + t;
@@ -313,10 +312,10 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
             const uint4 v = *(const uint4*)&tileT[c * (CAST_TILE / 4) + 4 * qsw];
             const int64_t gc = c0 + c;
             const int64_t gr = r0 + 16 * q;
-            if (gc < cols && gr < rows) {
-                // k-blocked: [rows/64][cols][64] (rows % 64 == 0, checked by the host)
+            if (gc < cols && (gr < rows || out_t_kb == F8MI_LAYOUT_KBLOCK64_PAD128)) {
+                // k-blocked: [rows/64][cols][64] (rows % 64 == 0 or padded to it: the sixteen rows are always whole)
                 uint8_t* dst = out_t_kb ? out_t + ((gr >> 6) * cols + gc) * 64 + (gr & 63) : out_t + gc * rows + gr;
-                if (t_vec) {  // rows % 16 == 0 implies gr + 16 <= rows
+                if (out_t_kb || gr + 16 <= rows) {
                     store16(dst, v);
                 } else {
                     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -349,7 +348,7 @@ constexpr int SMALL_THREADS = 1024;
 constexpr int SMALL_ITEMS_PER_THREAD = 4;
 constexpr int64_t SMALL_MAX_ITEMS = (int64_t)SMALL_THREADS * SMALL_ITEMS_PER_THREAD;  // 32 K elements: 64 KB of bf16
 
-template <int DT, int FMT, bool VEC>
+template <int DT, int FMT>
 __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
                                                                            int64_t ld, float* __restrict__ scale_out,
                                                                            uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
@@ -364,7 +363,7 @@ __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const
     for (int u = 0; u < SMALL_ITEMS_PER_THREAD; u++) {
         const int64_t it = t + (int64_t)u * SMALL_THREADS;
         // past the last item: row == rows, which load_row8 reads as zeros
-        load_row8<DT, VEC>(r[u], x, it < items ? it / groups : rows, (it % groups) * 8, rows, cols, ld);
+        load_row8<DT>(r[u], x, it < items ? it / groups : rows, (it % groups) * 8, rows, cols, ld);
     }
 #pragma unroll
     for (int u = 0; u < SMALL_ITEMS_PER_THREAD; u++) m = absmax_row<DT>(r[u], m);
@@ -381,7 +380,6 @@ __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const
     const float scale = amax_to_scale_dev(abs_bits_to_float(amax_bits, DT), DT, FMT, DT == F8MI_FP16);
     if (t == 0) *scale_out = scale;
     constexpr float fmax = FMT == F8MI_E4M3FN ? 448.0f : 57344.0f;
-    const bool out_vec = (cols % 8 == 0) && ((uintptr_t)out % 8 == 0);
 #pragma unroll
     for (int u = 0; u < SMALL_ITEMS_PER_THREAD; u++) {
         const int64_t it = t + (int64_t)u * SMALL_THREADS;
@@ -393,8 +391,8 @@ __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const
         const uint32_t lo = cvt4_fp8<FMT>(f[0], f[1], f[2], f[3]), hi = cvt4_fp8<FMT>(f[4], f[5], f[6], f[7]);
         if (out) {
             uint8_t* p = out_kb ? out + ((col >> 6) * rows + row) * 64 + (col & 63) : out + row * cols + col;
-            if (out_vec) {
-                *(uint2*)p = make_uint2(lo, hi);
+            if (col + 8 <= cols) {
+                store8_any(p, lo, hi);
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; i++)
@@ -415,16 +413,11 @@ __global__ __launch_bounds__(SMALL_THREADS) void cast_dynamic_small_kernel(const
 }
 
 template <int DT>
-static int launch_cast_small(int fmt, bool vec, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
+static int launch_cast_small(int fmt, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
                              float* scale_dev, uint8_t* out, uint8_t* out_t, int out_kb, int out_t_kb) {
     const dim3 g(1), b(SMALL_THREADS);
-    if (fmt == F8MI_E4M3FN) {
-        if (vec) hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E4M3FN, true>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
-        else hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E4M3FN, false>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
-    } else {
-        if (vec) hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E5M2, true>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
-        else hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E5M2, false>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
-    }
+    if (fmt == F8MI_E4M3FN) hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E4M3FN>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+    else hipLaunchKernelGGL((cast_dynamic_small_kernel<DT, F8MI_E5M2>), g, b, 0, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
     return check_hip(hipGetLastError(), "cast (dynamic, one workgroup) kernel launch");
 }
 
@@ -440,20 +433,19 @@ __global__ void cast_zero_amax_kernel(float* amax_out) {
 }
 
 template <int DT, int PROD, int FMT>
-static int launch_cast2(bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
+static int launch_cast2(dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
                         const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb,
                         const AmaxSource& src) {
-    if (vec) hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, true>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src.ws, src.nblocks, src.scale_out);
-    else hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT, false>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src.ws, src.nblocks, src.scale_out);
+    hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src.ws, src.nblocks, src.scale_out);
     return check_hip(hipGetLastError(), "cast kernel launch");
 }
 
 template <int DT, int PROD>
-static int launch_cast1(int fmt, bool vec, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols,
+static int launch_cast1(int fmt, dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols,
                         int64_t ld, const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev,
                         int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb, const AmaxSource& src) {
-    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
-    return launch_cast2<DT, PROD, F8MI_E5M2>(vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+    if (fmt == F8MI_E4M3FN) return launch_cast2<DT, PROD, F8MI_E4M3FN>(g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+    return launch_cast2<DT, PROD, F8MI_E5M2>(g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
 }
 
 // Validates and launches the cast.  `src.ws` null: the scale is read from scale_dev (f8mi_cast_layout).  Not null
@@ -462,10 +454,11 @@ static int launch_cast1(int fmt, bool vec, dim3 g, hipStream_t stream, const voi
 static int cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
                             int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
                             float* amax_dev, hipStream_t stream, const AmaxSource& src) {
-    if ((out_layout != F8MI_LAYOUT_ROWMAJOR && out_layout != F8MI_LAYOUT_KBLOCK64) || (out_t_layout != F8MI_LAYOUT_ROWMAJOR && out_t_layout != F8MI_LAYOUT_KBLOCK64)) { set_error("f8mi_cast: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
-    if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
-    if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
-    const int out_kb = out_layout == F8MI_LAYOUT_KBLOCK64, out_t_kb = out_t_layout == F8MI_LAYOUT_KBLOCK64;
+    if (out_layout < F8MI_LAYOUT_ROWMAJOR || out_layout > F8MI_LAYOUT_KBLOCK64_PAD128 || out_t_layout < F8MI_LAYOUT_ROWMAJOR || out_t_layout > F8MI_LAYOUT_KBLOCK64_PAD128) { set_error("f8mi_cast: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
+    if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast: k-blocked `out` needs cols %% 64 == 0 (cols=%lld); F8MI_LAYOUT_KBLOCK64_PAD128 takes any", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
+    if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld); F8MI_LAYOUT_KBLOCK64_PAD128 takes any", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
+    // the kernel takes the layout codes as they are (0: row-major, otherwise k-blocked; PAD128: whole tiles are written)
+    const int out_kb = out ? out_layout : F8MI_LAYOUT_ROWMAJOR, out_t_kb = out_t ? out_t_layout : F8MI_LAYOUT_ROWMAJOR;
     // ld == 0: every row reads the same `cols` elements (the kernels address row * ld + col)
     if (rows < 0 || cols < 0 || (ld < cols && ld != 0)) { set_error("f8mi_cast: bad shape rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld); return F8MI_ERR_INVALID_ARG; }
     if (in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast: unknown dtype/format code"); return F8MI_ERR_INVALID_ARG; }
@@ -485,7 +478,6 @@ static int cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t l
     dim3 g((unsigned)(tx * ty));
     const int64_t tiles_x = tx, tiles_y = ty;
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
-    const bool vec = ((uintptr_t)x % 16 == 0) && ((ld * esz) % 16 == 0);
     if (amax_dev) {
         hipLaunchKernelGGL(cast_zero_amax_kernel, dim3(1), dim3(64), 0, stream, amax_dev);
         int rc = check_hip(hipGetLastError(), "cast_zero_amax_kernel");
@@ -494,14 +486,14 @@ static int cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t l
     const double n = (double)rows * (double)cols;
     ProfScope prof(F8MI_K_CAST, (ld == 0 ? (double)cols : n) * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
     if (in_dtype == F8MI_BF16) {
-        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
-        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
     }
     if (in_dtype == F8MI_FP16) {
-        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
-        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
     }
-    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, vec, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
 }
 
 }  // namespace f8mi
@@ -530,17 +522,17 @@ extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int6
     if (rows < 0 || cols < 0 || (ld < cols && ld != 0) || in_dtype < 0 || in_dtype > 2 || fp8_fmt < 0 || fp8_fmt > 1) { set_error("f8mi_cast_dynamic: bad shape or dtype/format code"); return F8MI_ERR_INVALID_ARG; }
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
     const int64_t n = rows * cols;
-    if (n > 0 && rows * ((cols + 7) / 8) <= SMALL_MAX_ITEMS && (out || out_t)) {
+    const bool padded = (out && out_layout == F8MI_LAYOUT_KBLOCK64_PAD128) || (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64_PAD128);  // the tile kernel writes the padding
+    if (n > 0 && rows * ((cols + 7) / 8) <= SMALL_MAX_ITEMS && (out || out_t) && !padded) {
         if ((out_layout != F8MI_LAYOUT_ROWMAJOR && out_layout != F8MI_LAYOUT_KBLOCK64) || (out_t_layout != F8MI_LAYOUT_ROWMAJOR && out_t_layout != F8MI_LAYOUT_KBLOCK64)) { set_error("f8mi_cast_dynamic: unknown layout code"); return F8MI_ERR_INVALID_ARG; }
         if (out && out_layout == F8MI_LAYOUT_KBLOCK64 && cols % 64 != 0) { set_error("f8mi_cast_dynamic: k-blocked `out` needs cols %% 64 == 0 (cols=%lld)", (long long)cols); return F8MI_ERR_UNSUPPORTED; }
         if (out_t && out_t_layout == F8MI_LAYOUT_KBLOCK64 && rows % 64 != 0) { set_error("f8mi_cast_dynamic: k-blocked `out_t` needs rows %% 64 == 0 (rows=%lld)", (long long)rows); return F8MI_ERR_UNSUPPORTED; }
         if (!x) { set_error("f8mi_cast_dynamic: null tensor"); return F8MI_ERR_INVALID_ARG; }
-        const bool vec = ((uintptr_t)x % 16 == 0) && ((ld * esz) % 16 == 0);
         const int out_kb = out_layout == F8MI_LAYOUT_KBLOCK64, out_t_kb = out_t_layout == F8MI_LAYOUT_KBLOCK64;
         ProfScope prof(F8MI_K_CAST, (double)n * (esz + (out ? 1 : 0) + (out_t ? 1 : 0)), stream);
-        if (in_dtype == F8MI_BF16) return launch_cast_small<F8MI_BF16>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
-        if (in_dtype == F8MI_FP16) return launch_cast_small<F8MI_FP16>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
-        return launch_cast_small<F8MI_FP32>(fp8_fmt, vec, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+        if (in_dtype == F8MI_BF16) return launch_cast_small<F8MI_BF16>(fp8_fmt, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+        if (in_dtype == F8MI_FP16) return launch_cast_small<F8MI_FP16>(fp8_fmt, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
+        return launch_cast_small<F8MI_FP32>(fp8_fmt, stream, x, rows, cols, ld, scale_dev, out, out_t, out_kb, out_t_kb);
     }
     if (n == 0 || (!out && !out_t))  // only the scale is wanted
         return f8mi_amax_scale(x, rows, cols, ld, in_dtype, fp8_fmt, in_dtype, in_dtype == F8MI_FP16, nullptr, scale_dev, workspace, stream_);

@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/f8mi.h"
+#include "f8mi_knobs.h"
 
 namespace f8mi {
 
@@ -147,6 +148,19 @@ __device__ __forceinline__ uint4 load_nt16(const void* p) {
     u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+
+// 16- and 8-byte accesses at addresses aligned to the element size only (rows of a tensor whose row pitch is not a
+// multiple of 16 bytes).  Still one global_load / global_store instruction: gfx950 serves vector memory accesses at any
+// byte alignment, and the compiler emits the wide instruction for these under-aligned types.
+typedef u32x4 u32x4_any __attribute__((aligned(1)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x2 u32x2_any __attribute__((aligned(1)));
+__device__ __forceinline__ uint4 load_nt16_any(const void* p) {
+    u32x4 v = __builtin_nontemporal_load((const u32x4_any*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store16_any(void* p, uint4 v) { *(u32x4_any*)p = (u32x4){v.x, v.y, v.z, v.w}; }
+__device__ __forceinline__ void store8_any(void* p, uint32_t lo, uint32_t hi) { *(u32x2_any*)p = (u32x2){lo, hi}; }
 
 // Running maximum of sign-cleared 16-bit patterns, two per dword: `m` holds two independent 16-bit maxima
 // (v_and + v_pk_max_u16 per dword instead of five scalar operations); fold16 merges the halves at the end.

@@ -357,7 +357,7 @@ extern "C" int f8mi_gemm_nt_ws(const void* a, int a_fmt, int64_t lda, const void
     if (tiles_m * tiles_n > 0x7fffffff) { set_error("f8mi_gemm_nt: too many tiles"); return F8MI_ERR_UNSUPPORTED; }
     const bool aligned = ((uintptr_t)a % 16 == 0) && ((uintptr_t)bt % 16 == 0) && (lda % 16 == 0) && (ldb % 16 == 0);
     const int64_t csz = c_dtype == F8MI_FP32 ? 4 : 2;
-    const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
+    const int c_vec_ok = (uintptr_t)c % csz == 0;  // 16-byte stores at element alignment: any row pitch will do
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
     const uint8_t* A = (const uint8_t*)a;
@@ -413,7 +413,7 @@ extern "C" int f8mi_gemm_nt_kb_ws(const void* a, int a_fmt, const void* bt, int 
     const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7fffffff) { set_error("f8mi_gemm_nt_kb: too many tiles"); return F8MI_ERR_UNSUPPORTED; }
     const int64_t csz = c_dtype == F8MI_FP32 ? 4 : 2;
-    const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
+    const int c_vec_ok = (uintptr_t)c % csz == 0;  // 16-byte stores at element alignment: any row pitch will do
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
     const uint8_t* A = (const uint8_t*)a;
@@ -467,7 +467,7 @@ extern "C" int f8mi_gemm_kb_ex(const void* a, int a_fmt, int a_transposed, const
     const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7fffffff) { set_error("f8mi_gemm_kb_ex: too many tiles"); return F8MI_ERR_UNSUPPORTED; }
     const int64_t csz = c_dtype == F8MI_FP32 ? 4 : 2;
-    const int c_vec_ok = ((uintptr_t)c % 16 == 0) && ((ldc * csz) % 16 == 0);
+    const int c_vec_ok = (uintptr_t)c % csz == 0;  // 16-byte stores at element alignment: any row pitch will do
     dim3 g((unsigned)(tiles_m * tiles_n));
     ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
     // a transposed operand: 64 bytes between contraction rows, k * 64 between blocks of 64 rows

@@ -7,29 +7,6 @@ namespace f8mi {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// Compile-time knobs of the tile walk, for measurement builds (python _build.py --out other.so -DF8MI_WALK_GROUP=2,
-// loaded through F8MI_LIB); the shipped library is built with the defaults.
-#ifndef F8MI_WALK_GROUP
-#define F8MI_WALK_GROUP 4       // width of the bands the walk sweeps, in tiles
-#endif
-#ifndef F8MI_DMA_CACHE_POLICY   // cache-policy modifiers of the operand DMA (" nt", " sc1", ...), for measurement builds
-#define F8MI_DMA_CACHE_POLICY ""
-#endif
-#ifndef F8MI_WALK_XCD_CHUNK
-#define F8MI_WALK_XCD_CHUNK 0   // 0: each XCD owns one contiguous run of the tile order
-#endif
-#ifndef F8MI_WALK_SHORT_SIDE
-#define F8MI_WALK_SHORT_SIDE 0  // 1: sweep the bands along the shorter side of the tile grid
-#endif
-// Energy accounting, measurement builds only (the results are wrong): bit 0 leaves out the DMAs of the main loop (the
-// slabs keep the data of the first steps), bit 1 its LDS reads (the fragments of the first steps stay in registers),
-// bit 2 the barrier at the end of a step, bit 3 the wait and the barrier before the next step's fragments are read;
-// bit 4 makes every tile fetch the operands of the first tile (the same bytes into the LDS, nearly all of them L2 hits).
-// The rest stays, so the difference in time and in joules per flop is what the part left out costs.
-#ifndef F8MI_ABLATE
-#define F8MI_ABLATE 0
-#endif
-
 constexpr int SLAB_BYTES = 256 * 128;   // one operand, one step
 constexpr int HALF_BYTES = 256 * 64;    // one 64-deep unit of it
 constexpr int NSLAB_A = 3, NSLAB_B = 2;
@@ -126,7 +103,7 @@ struct Epilogue16 {
         if (row < M && col < N) {
             uint16_t* dst = (uint16_t*)C + (int64_t)row * ldc + col;
             if (c_vec_ok && col + 8 <= N) {
-                *(uint4*)dst = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                store16_any(dst, make_uint4(s0[0], s1[0], s0[1], s1[1]));
             } else {
                 const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
 #pragma unroll
@@ -165,7 +142,7 @@ __device__ __forceinline__ void store_c_tile16_fp32(v4f (&acc)[8][8], int m0, in
             for (int r = 0; r < 4; r++) v[r] = acc_read(acc[tj][ti][r]) * inv + bv[r];
             float* dst = Cf + (int64_t)row * ldc + col;
             if (c_vec_ok && col + 4 <= N) {
-                *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+                store16_any(dst, make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])));
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; r++)
@@ -245,7 +222,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
         tn = (lid % width) / gsz;
     }
     const int m0 = tm * BM, n0 = tn * BN;
-    const int fetch_m0 = (F8MI_ABLATE & 16) ? 0 : m0, fetch_n0 = (F8MI_ABLATE & 16) ? 0 : n0;
     // 1 / (sa * sb) for the epilogue, fetched now and kept in a scalar register: loaded after the main loop, the two
     // scales were a memory round trip with nothing to hide it
     const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
@@ -279,7 +255,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
             const int blk = min(m0 / 64 + (c >> 2), M / 64 - 1) - m0 / 64;  // blocks past the edge re-read the last one
             a_voff[d] = (uint32_t)(rowl * lda + blk * a_unit) + (c & 3) * 16;
         }
-        a_ptr = A + (int64_t)(fetch_m0 / 64) * a_unit;
+        a_ptr = A + (int64_t)(m0 / 64) * a_unit;
         a_step = 128 * lda;
     } else {
 #pragma unroll
@@ -287,7 +263,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
             const int r = (wave * 4 + i) * 16 + (lane >> 2);
             a_voff[i] = (uint32_t)(min(r, M - 1 - m0) * lda) + (((lane & 3) ^ (lane >> 5)) << 4);  // rows past the edge re-read the last row
         }
-        a_ptr = A + (int64_t)fetch_m0 * lda;
+        a_ptr = A + (int64_t)m0 * lda;
         a_step = 2 * a_unit;
     }
     if constexpr (B_TR) {
@@ -298,7 +274,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
             const int blk = min(n0 / 64 + (c >> 2), N / 64 - 1) - n0 / 64;
             b_voff[d] = (uint32_t)(rowl * ldb + blk * b_unit) + (c & 3) * 16;
         }
-        b_ptr = Bt + (int64_t)(fetch_n0 / 64) * b_unit;
+        b_ptr = Bt + (int64_t)(n0 / 64) * b_unit;
         b_step = 128 * ldb;
     } else {
 #pragma unroll
@@ -306,20 +282,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
             const int r = (wave * 4 + i) * 16 + (lane >> 2);
             b_voff[i] = (uint32_t)(min(r, N - 1 - n0) * ldb) + (((lane & 3) ^ (lane >> 5)) << 4);
         }
-        b_ptr = Bt + (int64_t)fetch_n0 * ldb;
+        b_ptr = Bt + (int64_t)n0 * ldb;
         b_step = 2 * b_unit;
     }
     uint32_t a_dst = 0, b_dst = 0;  // LDS address of the slabs being refilled
     // DMA d = 0..7 of this wave's share of a slab
-    bool main_loop = false;  // only read in builds with F8MI_ABLATE
     auto issue_a = [&](int d) __attribute__((always_inline)) {
-        if ((F8MI_ABLATE & 1) && main_loop) return;
         if constexpr (A_TR) dma16b(a_ptr, a_voff[d], a_dst + (wave * 8 + d) * 1024);
         else dma16b(d < 4 ? a_ptr : a_ptr + a_unit, a_voff[d & 3], a_dst + wave * 4096 + (d >> 2) * HALF_BYTES + (d & 3) * 1024);
         if (d == 7) a_ptr += a_step;
     };
     auto issue_b = [&](int d) __attribute__((always_inline)) {
-        if ((F8MI_ABLATE & 1) && main_loop) return;
         if constexpr (B_TR) dma16b(b_ptr, b_voff[d], b_dst + (wave * 8 + d) * 1024);
         else dma16b(d < 4 ? b_ptr : b_ptr + b_unit, b_voff[d & 3], b_dst + wave * 4096 + (d >> 2) * HALF_BYTES + (d & 3) * 1024);
         if (d == 7) b_ptr += b_step;
@@ -385,18 +358,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
 #pragma unroll
     for (int x = 0; x < 8; x++) fb[0][x] = frag_b(smem + NSLAB_A * SLAB_BYTES, x);
     fa[0] = frag_a(smem, 0);
-#if F8MI_ABLATE
-    fa[1] = frag_a(smem, 1);
-#pragma unroll
-    for (int x = 0; x < 8; x++) fb[1][x] = frag_b(smem + NSLAB_A * SLAB_BYTES, x ^ 1);
-#if F8MI_ABLATE & 1
-    a_dst = lds_u32 + 2 * SLAB_BYTES;  // the third slab of A holds step 2 (this moves a_ptr on: no fetch may follow)
-#pragma unroll
-    for (int d = 0; d < 8; d++) issue_a(d);
-#endif
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    main_loop = true;
-#endif
     lds_barrier();
 
     // One step t.  P: parity of t.  MODE 0: steps t+1 and t+2 exist (refills the slabs freed at this
@@ -425,7 +386,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
         if (MODE == 2 && EPI16) epi.load_bias_row();
 #pragma unroll
         for (int ti = 0; ti < 8; ti++) {
-            if (ti == 6 && MODE < 2 && !(F8MI_ABLATE & 8)) {
+            if (ti == 6 && MODE < 2) {
                 // this wave's DMAs of step t+1 have landed (the 12 of step t+2 issued so far may be in flight) ...
                 if (MODE == 0) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
                 else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -433,11 +394,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
             }
 #pragma unroll
             for (int tj = 0; tj < 8; tj++) {
-#if !(F8MI_ABLATE & 2)
                 if (tj == 0 && ti < 7) fa[(ti + 1) & 1] = frag_a(a_cur, ti + 1);
                 if (tj == 0 && ti == 7 && MODE < 2) fa[0] = frag_a(a_nxt, 0);
                 if (MODE < 2 && ti >= 6 && (tj & 1) == 1) fb[P ^ 1][(ti - 6) * 4 + (tj >> 1)] = frag_b(b_nxt, (ti - 6) * 4 + (tj >> 1));
-#endif
                 if (FIRST) mfma16_first<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
                 else mfma16<BF, AF>(acc[tj][ti], fb[P][tj], fa[ti & 1]);
                 F8MI_SCHED_FENCE();
@@ -455,7 +414,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nt_dma16_kernel(
                 }
             }
         }
-        if (MODE < 2 && !(F8MI_ABLATE & 4)) lds_barrier();  // step boundary: everybody is done with A of step t and has Bt of step t+1 in registers
+        if (MODE < 2) lds_barrier();  // step boundary: everybody is done with A of step t and has Bt of step t+1 in registers
         a_slab = a_next;
     };
 

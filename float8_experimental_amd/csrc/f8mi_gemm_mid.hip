@@ -185,7 +185,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
                 for (int e = 0; e < 4; e++) v[e] = acc[tj][ti][e] * inv + bv[e];
                 float* dst = (float*)C + ((int64_t)split * M + row) * ldc + col;
                 if (c_vec_ok && col + 4 <= N) {
-                    *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+                    store16_any(dst, make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])));
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++)
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_mid_kernel(
                 if (row < M && col < N) {
                     uint16_t* dst = (uint16_t*)C + (int64_t)row * ldc + col;
                     if (c_vec_ok && col + 8 <= N) {
-                        *(uint4*)dst = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                        store16_any(dst, make_uint4(s0[0], s1[0], s0[1], s1[1]));
                     } else {
                         const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
 #pragma unroll
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     if constexpr (C_DT == F8MI_FP32) {
         float* dst = (float*)C + row * ldc + col;
         if (c_vec_ok) {
-            *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+            store16_any(dst, make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])));
         } else {
 #pragma unroll
             for (int e = 0; e < 4; e++) dst[e] = v[e];
@@ -314,8 +314,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     } else {
         uint16_t* dst = (uint16_t*)C + row * ldc + col;
         const uint32_t p0 = pack2<C_DT>(v[0], v[1]), p1 = pack2<C_DT>(v[2], v[3]);
-        if (c_vec_ok) {  // rows start 16-byte aligned, col % 4 == 0: 8-byte aligned
-            *(uint2*)dst = make_uint2(p0, p1);
+        if (c_vec_ok) {  // one 8-byte store at element alignment
+            store8_any(dst, p0, p1);
         } else {
             dst[0] = (uint16_t)(p0 & 0xffffu); dst[1] = (uint16_t)(p0 >> 16);
             dst[2] = (uint16_t)(p1 & 0xffffu); dst[3] = (uint16_t)(p1 >> 16);

@@ -91,7 +91,7 @@ __device__ __forceinline__ void store_c_tile(v16f (&acc)[4][4], uint8_t* smem, i
                     }
                     float* dst = Cf + (int64_t)row * ldc + col;
                     if (c_vec_ok && col + 4 <= N) {
-                        *(float4*)dst = make_float4(v[0], v[1], v[2], v[3]);
+                        store16_any(dst, make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])));
                     } else {
 #pragma unroll
                         for (int r = 0; r < 4; r++)
@@ -137,7 +137,7 @@ __device__ __forceinline__ void store_c_tile(v16f (&acc)[4][4], uint8_t* smem, i
             if (row < M && col < N) {
                 uint16_t* dst = Ch + (int64_t)row * ldc + col;
                 if (c_vec_ok && col + 8 <= N) {
-                    *(uint4*)dst = v;
+                    store16_any(dst, v);
                 } else {
                     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll

@@ -70,7 +70,7 @@ class _DelayedBuffers:
 
 
 def _cast_for_gemm(t2d: torch.Tensor, float8_dtype, delayed: Optional[_DelayedBuffers], is_initialized: bool,
-                   want_row: bool, want_t: bool, row_kb: bool = False, t_kb: bool = False,
+                   want_row: bool, want_t: bool, row_kb: int = 0, t_kb: int = 0,
                    known_scale: Optional[torch.Tensor] = None):
     """fp8 copies of a 2-D tensor for the GEMMs: (as is, transposed, scale).
 
@@ -78,7 +78,8 @@ def _cast_for_gemm(t2d: torch.Tensor, float8_dtype, delayed: Optional[_DelayedBu
     float8_tensor.py:158-159 of the reference; one launch for a small tensor); delayed: first-iteration init if needed,
     then ONE launch that casts with the existing scale and records this step's amax
     (float8_scaling_utils.py:65-125).  ``row_kb`` / ``t_kb`` ask for the k-blocked layout
-    of the respective copy (same bytes, placed [k/64][rows][64] for the GEMM that contracts it).
+    of the respective copy (same bytes, placed [k/64][rows][64] for the GEMM that contracts it;
+    ``_native.KBLOCK_PAD``: with the contraction zero-padded to a multiple of 128).
     ``known_scale`` (dynamic scaling only): a scale computed beforehand for exactly this tensor
     (``precompute_float8_dynamic_scale_for_fsdp``); the amax pass is skipped.
     """
@@ -109,7 +110,9 @@ class _float8_linear_fn(torch.autograd.Function):
     its own last dimension, and the two GEMMs that use it read that one copy -- as it is where its last
     dimension is contracted, through LDS transpose loads where it is not (``f8mi_gemm_kb_ex``): no
     transposed fp8 copies exist.  Otherwise the cast writes the tensor and its transpose, each k-blocked
-    where its GEMM's contraction allows it (a multiple of 64, at least 384) and row-major where not.
+    for its GEMM's contraction -- as it is when that is a multiple of 64, zero-padded to a multiple of 128
+    when it is not (ragged layers: the reference pads the inner dimension for torch._scaled_mm the same way,
+    float8_utils.py:206-247) -- and row-major only where the contraction is short.
     """
 
     @staticmethod
@@ -130,9 +133,9 @@ class _float8_linear_fn(torch.autograd.Function):
             ctx.kb = None
             ctx.save_for_backward(x8, w8, sx, sw)
         else:
-            kb_fwd = not emulate and _native.kblock_ok(k)      # y = x W^T contracts in_features
-            kb_dx = not emulate_bw and _native.kblock_ok(n)    # dx = dy W contracts out_features
-            kb_dw = not emulate_bw and _native.kblock_ok(m)    # dw = dy^T x contracts tokens
+            kb_fwd = 0 if emulate else _native.kblock_layout(k)      # y = x W^T contracts in_features
+            kb_dx = 0 if emulate_bw else _native.kblock_layout(n)    # dx = dy W contracts out_features
+            kb_dw = 0 if emulate_bw else _native.kblock_layout(m)    # dw = dy^T x contracts tokens
             x8, x8t, sx = _cast_for_gemm(x2, e4m3_dtype, dl("input"), is_amax_initialized, True, need_dw, kb_fwd, kb_dw)
             w8, w8t, sw = _cast_for_gemm(weight, e4m3_dtype, dl("weight"), is_amax_initialized, True, need_dx, kb_fwd, kb_dx,
                                           known_scale=mod._precomputed_weight_scale)

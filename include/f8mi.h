@@ -54,6 +54,11 @@ extern "C" {
 int f8mi_version(void);
 const char* f8mi_last_error(void);
 
+/* "" for the library as shipped.  A measurement build (compiled with one of the knobs of csrc/f8mi_knobs.h set: another
+ * tile walk, cache policy, ...) answers with the knobs' names and values, so that callers and benchmarks can tell
+ * and record which build they run.  Every knob leaves results unchanged.  No counterpart in the reference. */
+const char* f8mi_build_knobs(void);
+
 /* Fills CU count, LDS bytes per workgroup and the gcn arch name of HIP device `device`.
  * Returns F8MI_ERR_ARCH when it is not a gfx950. */
 int f8mi_device_info(int device, int* cu_count, int* lds_bytes, char* arch, int arch_len);
@@ -161,10 +166,23 @@ int f8mi_gemm_nt(const void* a, int a_fmt, int64_t lda, const void* bt, int b_fm
  */
 #define F8MI_LAYOUT_ROWMAJOR 0
 #define F8MI_LAYOUT_KBLOCK64 1
+/* The same layout for ANY contraction length: the contraction is extended with zero bytes to f8mi_padded_k(kc), the
+ * next multiple of 128, and stored [f8mi_padded_k(kc)/64][R][64].  Zeros add nothing to a product, so a GEMM over the
+ * padded length gives the product of the unpadded operands -- what the reference's pad_tensor_for_matmul does to the
+ * inner dimension of a ragged layer before torch._scaled_mm (float8_utils.py:206-247, float8_ops.py:139-149), here
+ * done by the cast kernel as it writes the copy.  Output only: the GEMM entry points take such an operand as an
+ * ordinary k-blocked one of contraction length f8mi_padded_k(kc). */
+#define F8MI_LAYOUT_KBLOCK64_PAD128 2
+
+/* Contraction length of a F8MI_LAYOUT_KBLOCK64_PAD128 operand: k rounded up to a multiple of 128 (pure arithmetic). */
+int64_t f8mi_padded_k(int64_t k);
 
 /* f8mi_cast with a layout per output.  out_layout = KBLOCK64 stores `out` as [cols/64][rows][64]
  * (needs cols % 64 == 0), out_t_layout = KBLOCK64 stores the transpose as [rows/64][cols][64]
- * (needs rows % 64 == 0).  Everything else as f8mi_cast. */
+ * (needs rows % 64 == 0).  KBLOCK64_PAD128 takes any shape: `out` is [f8mi_padded_k(cols)/64][rows][64] and `out_t`
+ * [f8mi_padded_k(rows)/64][cols][64] bytes, every byte of which is written (zeros past the tensor's edge, also
+ * when the scale is NaN).  The input's rows need no alignment beyond the element's own: eight elements are one
+ * 16-byte load at any row pitch.  Everything else as f8mi_cast. */
 int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
                      int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
                      float* amax_dev, void* stream);

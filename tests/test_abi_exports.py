@@ -130,3 +130,31 @@ def test_gemm_plan_names_the_kernel_each_shape_class_takes():
     assert plan(4096, 4096, 448)[0] == "tiles256_mfma32" and plan(4096, 4096, 200)[0] == "staged"
     assert plan(4096, 4096, 4096, aligned=False)[0] == "staged" and plan(64, 4096, 4096, aligned=False)[0] == "staged"
     assert plan(0, 4096, 4096) == (None, 0, 0)
+
+
+def test_ragged_layers_stay_off_the_register_staged_gemm():
+    """The padding benchmark's shapes (reference benchmarks/bench_padding.py:117-132: dimensions that are no multiple
+    of 16) and the stress configuration's two layers: on the fused route every product whose contraction reaches 384
+    once padded runs on zero-padded k-blocked copies, i.e. on the LDS-DMA kernels, not on the register-staged one."""
+    from float8_experimental_amd import _native as nat
+
+    assert nat.lib().f8mi_padded_k(4097) == 4224 == nat.padded_k(4097) and nat.padded_k(128) == 128 and nat.padded_k(0) == 0
+    assert nat.kblock_layout(8192) == nat.KBLOCK and nat.kblock_layout(448) == nat.KBLOCK
+    assert nat.kblock_layout(4097) == nat.KBLOCK_PAD and nat.kblock_layout(1000) == nat.KBLOCK_PAD and nat.kblock_layout(257) == nat.KBLOCK_PAD
+    assert nat.kblock_layout(256) == nat.ROWMAJOR and nat.kblock_layout(200) == nat.ROWMAJOR
+    shapes = [(4099, 4097, 11007), (4099, 1000, 3000)]                                  # (tokens, in, out): config 5
+    shapes += [(8193, 2501, 5008), (65, 253, 4096), (1023, 1029, 2512), (4095, 511, 10000), (2047, 3073, 8192),
+               (511, 769, 7504), (127, 4097, 12288), (32769, 15, 15024), (9217, 8191, 20480),
+               (16385, 1025, 25008)]                                                     # (M, K, N) of the padding benchmark
+    for m, k, n in shapes:
+        route = nat.linear_route(m, k, n)
+        for name in ("output", "grad_input", "grad_weight"):
+            layout, kc, (kernel, parts, mid) = route[name]
+            short = {"output": k, "grad_input": n, "grad_weight": m}[name] <= 256
+            if short:
+                assert layout == nat.ROWMAJOR
+                continue
+            assert layout in (nat.KBLOCK, nat.KBLOCK_PAD) and kc % 128 in (0, 64), (m, k, n, name, route[name])
+            assert kernel != "staged", (m, k, n, name, route[name])
+    # the layers of the benchmark keep one fp8 copy per tensor
+    assert nat.linear_route(16384, 8192, 10240)["one_copy"] and not nat.linear_route(4099, 4097, 11007)["one_copy"]

@@ -272,6 +272,68 @@ def test_cast_kblocked_refused_by_the_library_when_not_a_multiple_of_64(nat):
     assert rc != 0
 
 
+def _unblock(t_kb):
+    """[kc/64, rows, 64] k-blocked bytes -> [rows, kc] row-major (numpy)."""
+    b = fp8_bytes(t_kb)
+    return b.transpose(1, 0, 2).reshape(b.shape[1], b.shape[0] * 64)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(1, 1), (33, 47), (128, 128), (257, 131), (130, 1000), (1000, 136), (4099, 1000), (200, 4097),
+                                   (3, 50, 70)])
+def test_cast_zero_padded_kblocked_layout(nat, dt, shape):
+    """F8MI_LAYOUT_KBLOCK64_PAD128 takes any shape: the output holds the row-major result's bytes, k-blocked after the
+    contraction has been extended to a multiple of 128, and every byte of the extension is zero -- with a dynamic
+    scale, a delayed one (amax fused), for both fp8 formats, for rows at an unaligned pitch, and under a NaN scale."""
+    co, to = _oracles()
+    x = heavy(shape, TORCH_DT[dt], 11)
+    rows, cols = x.numel() // shape[-1], shape[-1]
+    rp, cp = nat.padded_k(rows), nat.padded_k(cols)
+    xd = x.to(DEV)
+
+    def check(out, out_t, want, what):
+        assert out.shape == (cp // 64, rows, 64) and out_t.shape == (rp // 64, cols, 64), what
+        o, t = _unblock(out), _unblock(out_t)
+        assert np.array_equal(o[:, :cols], want) and not o[:, cols:].any(), what
+        assert np.array_equal(t[:, :rows], want.T) and not t[:, rows:].any(), what
+
+    for fmt, (code, tdt) in F8.items():
+        s = to.tensor_to_scale(x, tdt)
+        want = fp8_bytes(to.cast_to_fp8(x, s, tdt)).reshape(rows, cols)
+        out, out_t, sc = nat.cast_dynamic(xd, tdt, want_out_t=True, out_kblock=nat.KBLOCK_PAD, out_t_kblock=nat.KBLOCK_PAD)
+        assert sc.item() == s.item()
+        check(out, out_t, want, (dt, fmt, shape, "dynamic"))
+        s1 = (s * 2.5).reshape(1)
+        amax = torch.full((1,), -1.0, dtype=torch.float32, device=DEV)
+        out, out_t = nat.cast(xd, s1.to(DEV), tdt, product_dtype=torch.float32, want_out_t=True, amax_out=amax,
+                              out_kblock=nat.KBLOCK_PAD, out_t_kblock=nat.KBLOCK_PAD)
+        check(out, out_t, fp8_bytes(to.cast_to_fp8(x, s1, tdt)).reshape(rows, cols), (dt, fmt, shape, "delayed"))
+        assert amax.item() == to.tensor_to_amax(x).float().item()
+    # one padded and one row-major output in the same call
+    tdt = torch.float8_e4m3fn
+    s = to.tensor_to_scale(x, tdt)
+    want = fp8_bytes(to.cast_to_fp8(x, s, tdt)).reshape(rows, cols)
+    out, out_t = nat.cast(xd, s.to(DEV), tdt, want_out_t=True, out_kblock=nat.KBLOCK_PAD)
+    assert np.array_equal(_unblock(out)[:, :cols], want) and np.array_equal(fp8_bytes(out_t), want.T)
+    out, out_t = nat.cast(xd, s.to(DEV), tdt, want_out_t=True, out_t_kblock=nat.KBLOCK_PAD)
+    assert np.array_equal(fp8_bytes(out).reshape(rows, cols), want) and np.array_equal(_unblock(out_t)[:, :rows], want.T)
+    # a NaN scale turns every element into a NaN code and leaves the padding zero
+    out, out_t = nat.cast(xd, torch.full((), float("nan"), device=DEV), tdt, want_out_t=True, out_kblock=nat.KBLOCK_PAD,
+                          out_t_kblock=nat.KBLOCK_PAD)
+    o, t = _unblock(out), _unblock(out_t)
+    assert ((o[:, :cols] & 0x7f) == 0x7f).all() and not o[:, cols:].any()
+    assert ((t[:, :rows] & 0x7f) == 0x7f).all() and not t[:, rows:].any()
+    # rows at a pitch that is no multiple of 16 bytes (a column slice of a wider tensor)
+    if x.dim() == 2 and cols > 9:
+        v, vd = x[:, 3:cols - 2], xd[:, 3:cols - 2]
+        s = to.tensor_to_scale(v, tdt)
+        want = fp8_bytes(to.cast_to_fp8(v, s, tdt)).reshape(rows, cols - 5)
+        out, out_t, sc = nat.cast_dynamic(vd, tdt, want_out_t=True, out_kblock=nat.KBLOCK_PAD, out_t_kblock=nat.KBLOCK_PAD)
+        o, t = _unblock(out), _unblock(out_t)
+        assert sc.item() == s.item() and np.array_equal(o[:, :cols - 5], want) and not o[:, cols - 5:].any()
+        assert np.array_equal(t[:, :rows], want.T) and not t[:, rows:].any()
+
+
 def test_cast_row_strided_and_c_oracle(nat):
     co, to = _oracles()
     base = heavy((70, 400), torch.bfloat16, 4)
@@ -671,6 +733,40 @@ def test_gemm_with_transposed_operands_equals_row_major_bitwise(nat, m, n, k):
             torch.testing.assert_close(got.float(), want.float(), rtol=2.0**-7, atol=1e-2)
     with pytest.raises(nat.Float8NativeError):
         nat.gemm_kb_ex(a_tr, True, sa, _to_kb(bt), False, sb, torch.bfloat16)
+
+
+def _to_kb_padded(t):
+    """[rows, k] fp8 -> zero-padded k-blocked [padded_k/64, rows, 64] and the row-major padded matrix (device)."""
+    rows, k = t.shape
+    kp = -(-k // 128) * 128
+    padded = torch.zeros(rows, kp, dtype=torch.uint8, device=t.device)
+    padded[:, :k] = t.view(torch.uint8)
+    return padded.view(rows, kp // 64, 64).permute(1, 0, 2).contiguous().view(t.dtype), padded.view(t.dtype)
+
+
+@pytest.mark.parametrize("m,n,k", [(300, 200, 385), (257, 511, 1000), (129, 77, 4097), (4099, 1000, 3000), (1000, 3000, 4099),
+                                   (64, 8190, 2047), (20, 515, 8191)])
+def test_gemm_on_zero_padded_kblocked_operands(nat, m, n, k):
+    """A ragged contraction on the LDS-DMA kernels: operands k-blocked with the contraction zero-padded to a multiple of
+    128 (what the cast writes with F8MI_LAYOUT_KBLOCK64_PAD128) give the bits of the row-major product over the padded
+    length, and the value of the unpadded product (register-staged kernel) within the accumulation tolerance.  n and
+    the row pitch of C are odd in most cases: C leaves in 16-byte stores at 2-byte alignment."""
+    a = _rand_fp8((m, k), torch.float8_e5m2, m + k, 4.0).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e4m3fn, n + k, 4.0).to(DEV)
+    sa, sb = torch.tensor(3.0, device=DEV), torch.tensor(0.5, device=DEV)
+    a_kb, a_pad = _to_kb_padded(a)
+    b_kb, b_pad = _to_kb_padded(bt)
+    bias = (torch.randn(n) * 3).to(torch.bfloat16).to(DEV)
+    for out_dt, b in ((torch.bfloat16, bias), (torch.float32, None), (torch.float16, None)):
+        got = nat.gemm_nt_kb(a_kb, sa, b_kb, sb, out_dt, bias=b, split_k=False)
+        want = nat.gemm_nt(a_pad, sa, b_pad, sb, out_dt, bias=b, split_k=False)
+        assert torch.equal(got, want), (m, n, k, out_dt)
+        ragged = nat.gemm_nt(a, sa, bt, sb, out_dt, bias=b, split_k=False).double()
+        bound = (a.float().abs() @ bt.float().abs().t()).double() / 1.5
+        eps_out = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-23}[out_dt]
+        tol = 2 * eps_out * ragged.abs() + 2.0**-12 * bound + 1e-30
+        assert ((got.double() - ragged).abs() <= tol).all(), (m, n, k, out_dt)
+    _gemm_check(nat, m, n, k, "e5m2", "e4m3", torch.bfloat16, seed=m + n + k)
 
 
 def test_gemm_kblocked_refuses_short_or_ragged_k(nat):
