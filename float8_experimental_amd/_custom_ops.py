@@ -50,7 +50,8 @@ def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, produc
     the reference (float8_tensor.py:158-159, float8_utils.py:123-139), optionally with the amax pass of delayed
     scaling (float8_scaling_utils.py:89) folded in.  ``product_dtype``: what ``x * scale`` is rounded to."""
     amax = torch.empty(1 if want_amax else 0, dtype=torch.float32, device=x.device)
-    bits, _ = _native.cast(x, scale, float8_dtype, product_dtype=product_dtype, amax_out=amax if want_amax else None)
+    with _native.transient_workspaces():
+        bits, _ = _native.cast(x, scale, float8_dtype, product_dtype=product_dtype, amax_out=amax if want_amax else None)
     return bits, amax
 
 

@@ -40,6 +40,8 @@ EXPORTS = (
     "f8mi_amax_tile_elems",
     "f8mi_cast",
     "f8mi_cast_layout",
+    "f8mi_cast_delayed",
+    "f8mi_delayed_workspace_bytes",
     "f8mi_cast_dynamic",
     "f8mi_cast_dynamic_static",
     "f8mi_gemm_nt",
@@ -98,6 +100,10 @@ def lib() -> C.CDLL:
         L.f8mi_cast.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, vp, fp, vp, vp]
         L.f8mi_cast_layout.restype = i32
         L.f8mi_cast_layout.argtypes = [vp, i64, i64, i64, i32, fp, i32, i32, vp, i32, vp, i32, fp, vp]
+        L.f8mi_delayed_workspace_bytes.restype = C.c_size_t
+        L.f8mi_delayed_workspace_bytes.argtypes = []
+        L.f8mi_cast_delayed.restype = i32
+        L.f8mi_cast_delayed.argtypes = [vp, i64, i64, i64, i32, fp, i32, vp, i32, vp, i32, fp, vp, vp]
         L.f8mi_cast_dynamic.restype = i32
         L.f8mi_cast_dynamic.argtypes = [vp, i64, i64, i64, i32, i32, fp, vp, i32, vp, i32, vp, vp]
         L.f8mi_cast_dynamic_static.restype = i32
@@ -212,6 +218,22 @@ def workspace(dev: torch.device) -> torch.Tensor:
     if ws is None:
         ws = torch.zeros(lib().f8mi_workspace_bytes() // 4, dtype=torch.int32, device=dev)
         _workspaces[key] = ws
+    return ws
+
+
+_delayed_workspaces = {}
+
+
+def delayed_workspace(dev: torch.device) -> torch.Tensor:
+    """The zeroed words f8mi_cast_delayed folds the amax into (and leaves zeroed), one per (device, stream)."""
+    _check_device(dev)
+    words = lib().f8mi_delayed_workspace_bytes() // 4
+    if getattr(_tls, "transient", False):
+        return torch.zeros(words, dtype=torch.int32, device=dev)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _raw_stream(dev))
+    ws = _delayed_workspaces.get(key)
+    if ws is None:
+        ws = _delayed_workspaces[key] = torch.zeros(words, dtype=torch.int32, device=dev)
     return ws
 
 
@@ -424,6 +446,13 @@ def cast(x: torch.Tensor, scale: torch.Tensor, float8_dtype: torch.dtype, produc
     if rows * cols == 0:  # nothing to convert (an empty batch); torch hands out null pointers for empty tensors
         if amax_out is not None:
             amax_out.zero_()
+        return out, out_t
+    if amax_out is not None and product_dtype == torch.float32:  # the delayed-scaling cast
+        rc = lib().f8mi_cast_delayed(xs.data_ptr(), rows, cols, ld, _DT[x.dtype], scale.data_ptr(), _F8[float8_dtype],
+                                     out.data_ptr() if out is not None else None, int(out_kblock),
+                                     out_t.data_ptr() if out_t is not None else None, int(out_t_kblock),
+                                     amax_out.data_ptr(), delayed_workspace(x.device).data_ptr(), _stream(x))
+        _check(rc, "f8mi_cast_delayed")
         return out, out_t
     rc = lib().f8mi_cast_layout(xs.data_ptr(), rows, cols, ld, _DT[x.dtype], scale.data_ptr(), _DT[product_dtype],
                                 _F8[float8_dtype], out.data_ptr() if out is not None else None, int(out_kblock),

@@ -36,10 +36,11 @@ __device__ __forceinline__ void store16(uint8_t* p, uint4 v) {
 }
 
 constexpr int CAST_THREADS = 256;
+constexpr int SPREAD_WORDS = 1024;  // words of the delayed-scaling workspace (f8mi_delayed_workspace_bytes)
 constexpr int CAST_TILE = 128;
 constexpr int CAST_GROUP = 8;
 
-// Fused amax of the cast kernel: *amax_out was zeroed by a tiny kernel launched just before, and holds the
+// Fused amax of the cast kernel, without a workspace: *amax_out was zeroed by a tiny kernel launched just before, and holds the
 // running maximum as an fp32 bit pattern (non-negative floats and NaNs order like unsigned integers).
 // No ticket and, for all but a handful of blocks, no atomic at all: the value only grows, so a block whose
 // maximum is not above a (possibly stale) read of it has nothing to add.  (Reducing and reading the word early, right
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
                                                             uint8_t* __restrict__ out, uint8_t* __restrict__ out_t,
                                                             float* amax_out, int64_t tiles_x, int64_t tiles_y,
                                                             int out_kb, int out_t_kb, const uint32_t* __restrict__ amax_ws,
-                                                            int amax_nblocks, float* scale_out) {
+                                                            int amax_nblocks, float* scale_out, uint32_t* amax_spread) {
     __shared__ uint32_t tileT[CAST_TILE * CAST_TILE / 4];  // [column][row/4] dwords, swizzled
     __shared__ uint32_t red[CAST_THREADS / 64];
 
@@ -327,7 +328,19 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_kernel(const void* __restri
         }
     }
 
-    if (amax_out) {
+    if (amax_out && amax_spread) {
+        // Every wave folds its maximum (the bit pattern in the input's dtype) into one of SPREAD_WORDS words with an
+        // atomic that returns nothing: no LDS, no barrier, no round trip to wait for, and a word sees about one atomic
+        // per (tiles * 4 / SPREAD_WORDS) waves, spread over the whole run of the kernel.  cast_spread_finalize_kernel
+        // turns the words into *amax_out.  (Measured per tensor of the benchmark, 128 MB .. 1.8 GB, against the cast
+        // without amax: folding into *amax_out itself, one compare-and-atomic per workgroup at its end as below, +6 ..
+        // +20 us -- the workgroup holds its LDS and wave slots for the round trip of that last read; this + 0 .. 2 us,
+        // plus 4 us for the finalize launch.)
+        m = wave_max_u32(m);
+        if ((t & 63) == 0 && m)
+            (void)__hip_atomic_fetch_max(&amax_spread[(blockIdx.x * (CAST_THREADS / 64) + (t >> 6)) & (SPREAD_WORDS - 1)], m,
+                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if (amax_out) {
         m = wave_max_u32(m);
         const int wave = t >> 6, lane = t & 63;
         if (lane == 0) red[wave] = m;
@@ -426,17 +439,33 @@ struct AmaxSource {
     const uint32_t* ws;
     int nblocks;
     float* scale_out;
+    uint32_t* spread;  // delayed scaling: the zeroed words the fused amax is folded into (null: straight into *amax_dev)
 };
 
 __global__ void cast_zero_amax_kernel(float* amax_out) {
     if (threadIdx.x == 0) *amax_out = 0.0f;
 }
 
+// Second half of the fused amax with a workspace: the maximum of the SPREAD_WORDS words becomes *amax_out (widened to
+// fp32) and every word goes back to zero, which is the state the next call expects.  One workgroup.
+__global__ __launch_bounds__(SPREAD_WORDS) void cast_spread_finalize_kernel(uint32_t* __restrict__ spread, float* __restrict__ amax_out, int in_dt) {
+    __shared__ uint32_t red[SPREAD_WORDS / 64];
+    uint32_t m = spread[threadIdx.x];
+    if (m) spread[threadIdx.x] = 0u;
+    m = wave_max_u32(m);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        m = wave_max_u32(threadIdx.x < SPREAD_WORDS / 64 ? red[threadIdx.x] : 0u);
+        if (threadIdx.x == 0) *amax_out = abs_bits_to_float(m, in_dt);
+    }
+}
+
 template <int DT, int PROD, int FMT>
 static int launch_cast2(dim3 g, hipStream_t stream, const void* x, int64_t rows, int64_t cols, int64_t ld,
                         const float* scale_dev, uint8_t* out, uint8_t* out_t, float* amax_dev, int64_t tiles_x, int64_t tiles_y, int out_kb, int out_t_kb,
                         const AmaxSource& src) {
-    hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src.ws, src.nblocks, src.scale_out);
+    hipLaunchKernelGGL((cast_kernel<DT, PROD, FMT>), g, dim3(CAST_THREADS), 0, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src.ws, src.nblocks, src.scale_out, src.spread);
     return check_hip(hipGetLastError(), "cast kernel launch");
 }
 
@@ -478,22 +507,26 @@ static int cast_layout_impl(const void* x, int64_t rows, int64_t cols, int64_t l
     dim3 g((unsigned)(tx * ty));
     const int64_t tiles_x = tx, tiles_y = ty;
     const size_t esz = in_dtype == F8MI_FP32 ? 4 : 2;
-    if (amax_dev) {
-        hipLaunchKernelGGL(cast_zero_amax_kernel, dim3(1), dim3(64), 0, stream, amax_dev);
-        int rc = check_hip(hipGetLastError(), "cast_zero_amax_kernel");
-        if (rc) return rc;
-    }
     const double n = (double)rows * (double)cols;
+    // every launch of this call: the cast and what a fused amax adds before or after it
     ProfScope prof(F8MI_K_CAST, (ld == 0 ? (double)cols : n) * esz + n * ((out ? 1 : 0) + (out_t ? 1 : 0)), stream);
+    if (amax_dev && !src.spread) {
+        hipLaunchKernelGGL(cast_zero_amax_kernel, dim3(1), dim3(64), 0, stream, amax_dev);
+        if (int rc = check_hip(hipGetLastError(), "cast_zero_amax_kernel")) return rc;
+    }
+    int rc;
     if (in_dtype == F8MI_BF16) {
-        if (product_dtype == F8MI_BF16) return launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
-        return launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        if (product_dtype == F8MI_BF16) rc = launch_cast1<F8MI_BF16, F8MI_BF16>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        else rc = launch_cast1<F8MI_BF16, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+    } else if (in_dtype == F8MI_FP16) {
+        if (product_dtype == F8MI_FP16) rc = launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+        else rc = launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+    } else {
+        rc = launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
     }
-    if (in_dtype == F8MI_FP16) {
-        if (product_dtype == F8MI_FP16) return launch_cast1<F8MI_FP16, F8MI_FP16>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
-        return launch_cast1<F8MI_FP16, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
-    }
-    return launch_cast1<F8MI_FP32, F8MI_FP32>(fp8_fmt, g, stream, x, rows, cols, ld, scale_dev, out, out_t, amax_dev, tiles_x, tiles_y, out_kb, out_t_kb, src);
+    if (rc || !(amax_dev && src.spread)) return rc;
+    hipLaunchKernelGGL(cast_spread_finalize_kernel, dim3(1), dim3(SPREAD_WORDS), 0, stream, src.spread, amax_dev, in_dtype);
+    return check_hip(hipGetLastError(), "cast_spread_finalize_kernel");
 }
 
 }  // namespace f8mi
@@ -504,7 +537,7 @@ extern "C" int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64
                                 const float* scale_dev, int product_dtype, int fp8_fmt, uint8_t* out, int out_layout,
                                 uint8_t* out_t, int out_t_layout, float* amax_dev, void* stream) {
     return cast_layout_impl(x, rows, cols, ld, in_dtype, scale_dev, product_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, amax_dev,
-                            (hipStream_t)stream, AmaxSource{nullptr, 0, nullptr});
+                            (hipStream_t)stream, AmaxSource{nullptr, 0, nullptr, nullptr});
 }
 
 extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev,
@@ -513,6 +546,17 @@ extern "C" int f8mi_cast(const void* x, int64_t rows, int64_t cols, int64_t ld, 
     (void)workspace;
     return f8mi_cast_layout(x, rows, cols, ld, in_dtype, scale_dev, product_dtype, fp8_fmt, out, F8MI_LAYOUT_ROWMAJOR, out_t,
                             F8MI_LAYOUT_ROWMAJOR, amax_dev, stream);
+}
+
+extern "C" size_t f8mi_delayed_workspace_bytes(void) { return SPREAD_WORDS * sizeof(uint32_t); }
+
+extern "C" int f8mi_cast_delayed(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev, int fp8_fmt,
+                                 uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout, float* amax_dev, void* workspace,
+                                 void* stream) {
+    if (!amax_dev) { set_error("f8mi_cast_delayed: null amax"); return F8MI_ERR_INVALID_ARG; }
+    if (!workspace || (uintptr_t)workspace % 4 != 0) { set_error("f8mi_cast_delayed: null or misaligned workspace"); return F8MI_ERR_INVALID_ARG; }
+    return cast_layout_impl(x, rows, cols, ld, in_dtype, scale_dev, F8MI_FP32, fp8_fmt, out, out_layout, out_t, out_t_layout, amax_dev,
+                            (hipStream_t)stream, AmaxSource{nullptr, 0, nullptr, (uint32_t*)workspace});
 }
 
 extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt, float* scale_dev,
@@ -550,7 +594,7 @@ extern "C" int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int6
         if (int rc = launch_amax_partials(x, rows, cols, ld, in_dtype, (uint32_t*)workspace, stream, &nblocks)) return rc;
     }
     return cast_layout_impl(x, rows, cols, ld, in_dtype, nullptr, in_dtype, fp8_fmt, out, out_layout, out_t, out_t_layout, nullptr, stream,
-                            AmaxSource{(const uint32_t*)workspace, nblocks, scale_dev});
+                            AmaxSource{(const uint32_t*)workspace, nblocks, scale_dev, nullptr});
 }
 
 namespace f8mi {

@@ -187,6 +187,22 @@ int f8mi_cast_layout(const void* x, int64_t rows, int64_t cols, int64_t ld, int 
                      int product_dtype, int fp8_fmt, uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout,
                      float* amax_dev, void* stream);
 
+/* Delayed scaling in one call: f8mi_cast_layout with the module's existing scale (the product x * scale in fp32, as
+ * with the [1]-shaped scale buffer), and *amax_dev = max|x| of this call -- hp_tensor_to_float8_delayed
+ * (float8_scaling_utils.py:65-96: amax_buffer.fill_(tensor_to_amax(x)), then the cast with the stale scale).
+ * Same bytes and the same amax as f8mi_cast_layout with amax_dev; what differs is how the amax leaves the cast kernel:
+ * there every workgroup compares with *amax_dev at its end (and holds its LDS and wave slots for that round trip:
+ * 6 - 20 us per tensor of 128 MB - 1.8 GB), here every wave folds its maximum into one of 1024 words of `workspace`
+ * with an atomic that returns nothing, and a one-workgroup launch reduces the words (4 us).
+ *   workspace   f8mi_delayed_workspace_bytes() of device memory, 4-byte aligned, ALL ZERO before the first call that
+ *               uses it; every call leaves it all zero again when its work completes.  Not to be shared by calls that
+ *               can overlap in time (one per stream), and not the workspace of f8mi_amax_scale, whose contents are
+ *               arbitrary. */
+size_t f8mi_delayed_workspace_bytes(void);
+int f8mi_cast_delayed(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, const float* scale_dev, int fp8_fmt,
+                      uint8_t* out, int out_layout, uint8_t* out_t, int out_t_layout, float* amax_dev, void* workspace,
+                      void* stream);
+
 /* Dynamic scaling in one call: scale = f8mi_amax_scale(x) in x's own dtype, then f8mi_cast_layout(x, scale) with the
  * product in x's dtype -- hp_tensor_to_float8_dynamic (float8_scaling_utils.py:33-62: tensor_to_scale, then
  * hp_tensor_and_scale_to_float8 with the 0-dim scale).  *scale_dev receives the scale.  A tensor of at most

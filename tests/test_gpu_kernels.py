@@ -3,6 +3,8 @@
 Bars: amax, scales and fp8 bytes bit-exact (NaN codes may differ in the sign
 bit); GEMM within a stated tolerance of the emulated fp32 product.
 """
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -270,6 +272,41 @@ def test_cast_kblocked_refused_by_the_library_when_not_a_multiple_of_64(nat):
     assert rc != 0
     rc = L.f8mi_cast_layout(x.data_ptr(), 100, 96, 96, 0, s.data_ptr(), 0, 0, out.data_ptr(), 7, None, 0, None, None)
     assert rc != 0
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+def test_delayed_cast_with_workspace_equals_the_cast_without(nat, dt):
+    """f8mi_cast_delayed folds the amax into the 1024 words of its workspace and a second launch reduces them: same bytes
+    and the same amax as f8mi_cast_layout with amax_dev, the oracle's amax (NaN, inf, all-zero and all-negative-zero
+    tensors included), and the workspace is all zero again after every call -- also on the next, smaller call."""
+    co, to = _oracles()
+    L = nat.lib()
+    assert L.f8mi_delayed_workspace_bytes() == 4096
+    tdt = torch.float8_e4m3fn
+    cases = [heavy((777, 1031), TORCH_DT[dt], 3), heavy((4, 8), TORCH_DT[dt], 4), heavy((2048, 4096), TORCH_DT[dt], 5),
+             torch.zeros(300, 200, dtype=TORCH_DT[dt]), -torch.zeros(130, 70, dtype=TORCH_DT[dt])]
+    nan = heavy((257, 513), TORCH_DT[dt], 6)
+    nan[100, 17] = float("nan")
+    inf = heavy((129, 257), TORCH_DT[dt], 7)
+    inf[5, 5] = float("-inf")
+    cases += [nan, inf]
+    ws = nat.delayed_workspace(torch.device(DEV))
+    for x in cases:
+        xd = x.to(DEV)
+        s1 = torch.tensor([1.7], device=DEV)
+        a_new = torch.full((1,), -1.0, device=DEV)
+        a_old = torch.full((1,), -1.0, device=DEV)
+        out, out_t = nat.cast(xd, s1, tdt, product_dtype=torch.float32, want_out_t=True, amax_out=a_new)   # f8mi_cast_delayed
+        o2 = torch.empty_like(out)
+        t2 = torch.empty_like(out_t)
+        rc = L.f8mi_cast_layout(xd.data_ptr(), x.shape[0], x.shape[1], x.shape[1], CODE_DT[dt], s1.data_ptr(), 2, 0, o2.data_ptr(), 0,
+                                t2.data_ptr(), 0, a_old.data_ptr(), None)
+        assert rc == 0
+        assert torch.equal(out.view(torch.uint8), o2.view(torch.uint8)) and torch.equal(out_t.view(torch.uint8), t2.view(torch.uint8))
+        want = to.tensor_to_amax(x).float()
+        for a in (a_new, a_old):
+            assert (math.isnan(a.item()) and math.isnan(want.item())) or a.item() == want.item(), (dt, tuple(x.shape), a.item(), want.item())
+        assert not ws.any().item(), "the workspace must be all zero after a call"
 
 
 def _unblock(t_kb):
