@@ -53,25 +53,46 @@ def gemm_traffic(m, scaling):
     return total, why
 
 
+def _cuda0_pci_bus_id():
+    """PCI address of torch's cuda:0 ("0000:c1:00.0"), or None when torch is not loaded / has no GPU."""
+    torch = sys.modules.get("torch")
+    try:
+        if torch is None or not torch.cuda.is_available():
+            return None
+        p = torch.cuda.get_device_properties(0)
+        return "%04x:%02x:%02x.0" % (p.pci_domain_id, p.pci_bus_id, p.pci_device_id)
+    except Exception:
+        return None
+
+
 class Telemetry:
     """Socket power and shader clock of the GPU while the timed region runs, sampled from sysfs by a host thread
     (reads of two small files every 5 ms; nothing on the launch path)."""
 
-    def __init__(self, period=0.005):
+    def __init__(self, period=0.005, pci_bus_id=None):
+        """``pci_bus_id`` ("0000:c1:00.0"): the card to sample; default: the PCI address of torch's cuda:0 when torch is
+        loaded and a GPU is there, else the first card with power telemetry."""
         import glob
         import threading
 
+        if pci_bus_id is None:
+            pci_bus_id = _cuda0_pci_bus_id()
         self.period = period
         self.power_w, self.sclk_mhz = [], []
         self.cap_w = None
         self._stop = threading.Event()
         self._thread = None
-        self.power_file = self.sclk_file = None
-        for dev in sorted(glob.glob("/sys/class/drm/card[0-9]*/device")):
+        self.power_file = self.sclk_file = self.card = None
+        cards = sorted(glob.glob("/sys/class/drm/card[0-9]*/device"))
+        if pci_bus_id:  # the sysfs entry is a link to the PCI device: .../0000:c1:00.0
+            mine = [d for d in cards if os.path.basename(os.path.realpath(d)).lower() == pci_bus_id.lower()]
+            cards = mine or cards
+        for dev in cards:
             hw = sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*", "power1_input"))
                         + glob.glob(os.path.join(dev, "hwmon", "hwmon*", "power1_average")))
             if hw and os.path.exists(os.path.join(dev, "pp_dpm_sclk")):
                 self.power_file, self.sclk_file = hw[0], os.path.join(dev, "pp_dpm_sclk")
+                self.card = os.path.basename(os.path.realpath(dev))
                 try:
                     self.cap_w = int(open(os.path.join(os.path.dirname(hw[0]), "power1_cap")).read()) / 1e6
                 except (OSError, ValueError):
@@ -108,6 +129,7 @@ class Telemetry:
             return None
         mean = lambda v: sum(v) / len(v) if v else None
         return {"source": "sysfs hwmon power1_input + pp_dpm_sclk, every %d ms over the timed region" % int(self.period * 1e3),
+                "card": self.card,
                 "samples": len(self.power_w), "socket_power_W_mean": mean(self.power_w), "socket_power_W_max": max(self.power_w),
                 "power_cap_W": self.cap_w, "sclk_MHz_mean": mean(self.sclk_mhz),
                 "sclk_MHz_min": min(self.sclk_mhz) if self.sclk_mhz else None,
@@ -129,6 +151,8 @@ def parse():
     p.add_argument("--mfma-order", type=int, default=0, choices=[0, 1, 2, 3],
                    help="register-only MFMA loop: which operand changes between consecutive instructions "
                         "(0 the first, as in the GEMM; 1 the second; 2 both; 3 neither for eight in a row)")
+    p.add_argument("--no-other-configs", action="store_true",
+                   help="leave out the configurations besides the headline one (profiler runs of the headline's kernels)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run one plain 1 GiB device-to-device copy (for scaling hardware byte counters of a profiler run)")
     return p.parse_args()
@@ -210,6 +234,8 @@ def probe_mfma(torch, random_data, iters=4000, operands=None, seconds=0.8, order
     while time.perf_counter() < t_end:
         vals.append(once())
     t = tele.stop() or {}
+    if not vals or any(v is None for v in vals):  # a failed probe call: no figure rather than a wrong one
+        return None
     out = {"TFLOP/s": sum(vals) / len(vals), "socket_power_W": t.get("socket_power_W_mean"), "sclk_MHz": t.get("sclk_MHz_mean")}
     if idle_w and out["socket_power_W"]:
         out["pJ_per_flop_above_idle"] = (out["socket_power_W"] - idle_w) / out["TFLOP/s"]
@@ -267,6 +293,145 @@ def vendor_scaled_mm(torch, _native, layers, m, flop_step, iters):
                 "per_gemm": per_gemm}
     except Exception as e:  # a product this torch build does not take
         return {"scaled_mm_TFLOP/s": None, "error": f"{type(e).__name__}: {str(e)[:160]}"}
+
+
+def _prof_window(torch, _native, fn, reps):
+    """Runs fn() reps times with the library's per-kernel HIP-event counters on; {kernel: (launches, ms, work)}."""
+    _native.prof_reset()
+    _native.prof_enable(True)
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    _native.prof_enable(False)
+    prof = {name: _native.prof_read(kid) for name, kid in (("amax", _native.K_AMAX), ("cast", _native.K_CAST),
+                                                           ("gemm", _native.K_GEMM), ("sync", _native.K_SYNC))}
+    _native.prof_reset()
+    return prof
+
+
+def _rates(prof, flop=None, reps=1):
+    """GEMM TFLOP/s (over ``flop`` algorithmic flop per repetition when given: padded products count their unpadded
+    work), cast / amax GB/s and fractions of the peaks, from a _prof_window record."""
+    out = {}
+    n, ms, work = prof["gemm"]
+    if ms > 0:
+        f = flop * reps if flop else work
+        out["gemm_TFLOP/s"] = f / ms / 1e9
+        out["gemm_frac_of_fp8_peak"] = f / ms / 1e9 / PEAK_FP8_TFLOPS
+        out["gemm_ms"] = ms / reps
+    for k in ("cast", "amax"):
+        n, ms, work = prof[k]
+        if ms > 0:
+            out[f"{k}_GB/s"] = work / ms / 1e6
+            out[f"{k}_frac_of_hbm_peak"] = work / ms / 1e6 / PEAK_HBM_GBS
+            out[f"{k}_ms"] = ms / reps
+    return out
+
+
+LLAMA3_8B_LINEARS = [  # (name, K, N) of the seven linears of one Llama-3-8B decoder layer (d 4096, ffn 14336, 8 KV heads)
+    ("wq", 4096, 4096), ("wk", 4096, 1024), ("wv", 4096, 1024), ("wo", 4096, 4096),
+    ("w1", 4096, 14336), ("w3", 4096, 14336), ("w2", 14336, 4096),
+]
+RAGGED_LAYERS = [(4099, 4097, 11007), (4099, 1000, 3000)]  # (tokens, K, N): no dimension a multiple of 16
+
+
+def other_configs(torch, f8, _native, layers, args):
+    """The benchmark configurations besides the headline one, each outside the headline's timed region and measured
+    the same way (wall clock over whole steps, kernel times from HIP events on the launch stream): delayed scaling of
+    all three tensors on the same four shapes with one sync per step, the sync kernel's latency at 12 and 240
+    (layer, tensor) entries, the seven linear shapes of a Llama-3-8B layer at 8192 tokens, and two ragged layers."""
+    dev = torch.device("cuda:0")
+    steps = max(2, args.steps)
+    out = {}
+    DEL = f8.CastConfig(f8.ScalingType.DELAYED)
+    delayed_cfg = f8.Float8LinearConfig(cast_config_input=DEL, cast_config_weight=DEL, cast_config_grad_output=DEL)
+
+    def fwd_bwd(mod, x, dy):
+        x.grad = None
+        mod.weight.grad = None
+        mod(x).backward(dy)
+
+    # ---- delayed scaling x3 on the headline's shapes (same weights, inputs and gradients), history 16, one sync per step
+    if args.scaling == "dynamic":
+        mods = [f8.Float8Linear.from_float(lay[3], config=delayed_cfg) for lay in layers]
+        model = torch.nn.ModuleList(mods)
+
+        def dstep():
+            f8.sync_float8_amax_and_scale_history(model)
+            for mod, lay in zip(mods, layers):
+                fwd_bwd(mod, lay[5], lay[6])
+
+        flop = sum(3 * 2.0 * lay[5].shape[0] * lay[1] * lay[2] for lay in layers)
+        sec = timed(torch, dstep, steps, 2)
+        prof = _prof_window(torch, _native, dstep, 2)
+        r = {"ms_per_step": sec * 1e3, "TFLOP/s": flop / sec / 1e12, "history_len": 16,
+             "what": "delayed scaling of input, weight and grad_output; sync_float8_amax_and_scale_history over the four "
+                     "layers, then fwd+bwd of each; the cast is the fused amax + cast (4 bytes moved per bf16 element incl. "
+                     "its finalize launch)"}
+        r.update(_rates(prof, reps=2))
+        n, ms, _ = prof["sync"]
+        r["sync_us_per_launch"] = ms / max(n, 1) * 1e3
+        r["sync_entries"] = 3 * len(mods)
+        out["delayed_llama70b"] = r
+        del mods, model
+
+    # ---- sync latency by number of (layer, tensor) entries: kernel time from HIP events, and the host's wall time per call
+    lat = {}
+    for n_layers in (4, 80):
+        small = torch.nn.ModuleList([f8.Float8Linear.from_float(torch.nn.Linear(64, 64, bias=False, device=dev, dtype=torch.bfloat16),
+                                                                config=delayed_cfg) for _ in range(n_layers)])
+        for mod in small:
+            mod.last_seen_input_dtype = torch.bfloat16
+        call = lambda: f8.sync_float8_amax_and_scale_history(small)
+        wall = timed(torch, call, 200, 20)
+        prof = _prof_window(torch, _native, call, 50)
+        n, ms, nbytes = prof["sync"]
+        lat[f"{3 * n_layers}_entries"] = {"kernel_us": ms / max(n, 1) * 1e3, "launches_per_call": n / 50,
+                                         "host_wall_us_per_call_back_to_back": wall * 1e6, "bytes": nbytes / max(n, 1)}
+        del small
+    out["sync_latency"] = lat
+
+    # ---- the seven linear shapes of a Llama-3-8B layer at 8192 tokens (dynamic scaling), fwd+bwd each
+    tokens = 8192
+    per, tot_flop, tot_sec, tot_prof = {}, 0.0, 0.0, None
+    for name, k, n in LLAMA3_8B_LINEARS:
+        lin = torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.bfloat16)
+        mod = f8.Float8Linear.from_float(lin)
+        x = torch.randn(tokens, k, device=dev, dtype=torch.bfloat16).requires_grad_()
+        dy = (torch.randn(tokens, n, device=dev) * 1e-2).to(torch.bfloat16)
+        flop = 3 * 2.0 * tokens * k * n
+        sec = timed(torch, lambda: fwd_bwd(mod, x, dy), 4 * steps, 3)
+        prof = _prof_window(torch, _native, lambda: fwd_bwd(mod, x, dy), 4)
+        per[name] = {"K": k, "N": n, "ms": sec * 1e3, "TFLOP/s": flop / sec / 1e12, **_rates(prof, flop, 4)}
+        tot_flop += flop
+        tot_sec += sec
+        tot_prof = prof if tot_prof is None else {kk: tuple(a + b for a, b in zip(tot_prof[kk], prof[kk])) for kk in prof}
+        del lin, mod, x, dy
+    out["llama3_8b_linear_shapes"] = {"tokens": tokens, "ms_all_seven": tot_sec * 1e3, "TFLOP/s": tot_flop / tot_sec / 1e12,
+                                      **_rates(tot_prof, tot_flop, 4), "per_shape": per}
+
+    # ---- ragged layers (no dimension a multiple of 16): zero-padded k-blocked fp8 copies, fwd+bwd, against bf16
+    rag = {}
+    for tokens, k, n in RAGGED_LAYERS:
+        lin = torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.bfloat16)
+        mod = f8.Float8Linear.from_float(lin)
+        x = torch.randn(tokens, k, device=dev, dtype=torch.bfloat16).requires_grad_()
+        dy = (torch.randn(tokens, n, device=dev) * 1e-2).to(torch.bfloat16)
+        flop = 3 * 2.0 * tokens * k * n
+        sec = timed(torch, lambda: fwd_bwd(mod, x, dy), 10 * steps, 5)
+        prof = _prof_window(torch, _native, lambda: fwd_bwd(mod, x, dy), 10)
+        r = {"ms": sec * 1e3, "TFLOP/s": flop / sec / 1e12, **_rates(prof, flop, 10),
+             # a layer this small is bound by the host in eager mode (about 12 launches per fwd+bwd): the kernels' own time
+             "kernel_ms_sum": sum(prof[kk][1] for kk in ("amax", "cast", "gemm")) / 10,
+             "kernels": {p: list(_native.linear_route(tokens, k, n)[p][2]) for p in ("output", "grad_input", "grad_weight")}}
+        if not args.no_bf16:
+            secb = timed(torch, lambda: fwd_bwd(lin, x, dy), 10 * steps, 5)
+            r["bf16_ms"] = secb * 1e3
+            r["speedup_vs_bf16"] = secb / sec
+        rag[f"{tokens}x{k}->{n}"] = r
+        del lin, mod, x, dy
+    out["ragged_layers"] = rag
+    return out
 
 
 def cpu_baseline(torch, target_s):
@@ -389,6 +554,8 @@ def main():
         one_sync = (lambda: f8.sync_float8_amax_and_scale_history(lay[4])) if sync is not None else None
         t = timed(torch, lambda: step([lay], sync=one_sync), max(2, args.steps // 2), 1)
         per_shape[name] = {"fp8_ms": t * 1e3, "fp8_TFLOP/s": flop_per_shape[name] / t / 1e12}
+        # this shape's own kernels (the hbm_kernels figures above average over tensors of 134 MB to 1.9 GB)
+        per_shape[name].update(_rates(_prof_window(torch, _native, lambda: step([lay], sync=one_sync), 2), reps=2))
     bf16_step = None
     if not args.no_bf16:
         for lay in layers:
@@ -489,6 +656,9 @@ def main():
         "per_shape": per_shape,
         "frac_of_fp8_peak_end_to_end": flop_step / sec_step / 1e12 / PEAK_FP8_TFLOPS,
     }
+    out["library_build_knobs"] = _native.build_knobs()  # "" = the library as shipped
+    if not args.no_other_configs:
+        out["other_configs"] = other_configs(torch, f8, _native, layers, args)
     if bf16_step:
         out["bf16_linear"] = {"ms_per_step": bf16_step * 1e3, "TFLOP/s": flop_step / bf16_step / 1e12,
                               "speedup_fp8_over_bf16": bf16_step / sum(v["fp8_ms"] * 1e-3 for v in per_shape.values())}

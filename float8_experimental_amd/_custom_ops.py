@@ -75,6 +75,21 @@ def _(a, a_scale, bt, b_scale, out_dtype, bias):
     return torch.empty((a.shape[0], bt.shape[0]), dtype=out_dtype, device=a.device)
 
 
+@torch.library.custom_op("f8mi::scaled_mm", mutates_args=())
+def scaled_mm(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: torch.Tensor, out_dtype: torch.dtype,
+              bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``(a @ b) / (a_scale * b_scale) (+ bias)`` for fp8 operands in whatever layout they have: ``torch._scaled_mm`` as
+    the reference calls it (float8_python_api.py:24-64) without the layout rule that makes float8_ops.preprocess_addmm
+    copy (float8_ops.py:150-153) -- a row-major second operand is read transposed by the kernel where it can."""
+    with _native.transient_workspaces():
+        return _native.scaled_mm(a, a_scale, b, b_scale, out_dtype, bias=bias)
+
+
+@scaled_mm.register_fake
+def _(a, a_scale, b, b_scale, out_dtype, bias):
+    return torch.empty((a.shape[0], b.shape[1]), dtype=out_dtype, device=a.device)
+
+
 # ---- the fused linear ----------------------------------------------------------------------------------------
 
 

@@ -47,6 +47,7 @@ EXPORTS = (
     "f8mi_gemm_nt",
     "f8mi_gemm_nt_kb",
     "f8mi_gemm_kb_ex",
+    "f8mi_gemm_ex",
     "f8mi_sync",
     "f8mi_sync_host",
     "f8mi_delayed_init",
@@ -112,6 +113,8 @@ def lib() -> C.CDLL:
         L.f8mi_gemm_nt_kb.argtypes = [vp, i32, vp, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_kb_ex.restype = i32
         L.f8mi_gemm_kb_ex.argtypes = [vp, i32, i32, vp, i32, i32, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
+        L.f8mi_gemm_ex.restype = i32
+        L.f8mi_gemm_ex.argtypes = [vp, i32, i32, i64, vp, i32, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_nt.restype = i32
         L.f8mi_gemm_nt.argtypes = [vp, i32, i64, vp, i32, i64, i64, i64, i64, fp, fp, vp, i32, i64, vp, vp]
         L.f8mi_gemm_nt_ws.restype = i32
@@ -603,6 +606,49 @@ def gemm_nt(a: torch.Tensor, a_scale: torch.Tensor, bt: torch.Tensor, b_scale: t
                                bias.data_ptr() if bias is not None else None, ws, ws_bytes, _stream(a))
     _check(rc, "f8mi_gemm_nt_ws")
     return out
+
+
+ERR_UNSUPPORTED = -2  # F8MI_ERR_UNSUPPORTED
+
+
+def scaled_mm(a: torch.Tensor, a_scale: torch.Tensor, b: torch.Tensor, b_scale: torch.Tensor, out_dtype: torch.dtype,
+              bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``(a @ b) / (a_scale * b_scale) (+ bias)`` for fp8 ``a`` [m, k] and ``b`` [k, n] in ANY layout: what
+    ``torch._scaled_mm`` computes, without its rule that ``a`` be row-major and ``b`` column-major.  Row-major ``b``
+    (and column-major ``a`` next to it) are read transposed by the kernel where it can (f8mi_gemm_ex); where it
+    cannot -- small or ragged products -- the operand is copied into the layout ``gemm_nt`` takes, which is the copy
+    the reference always makes (float8_ops.py:150-153).  Same bits either way."""
+    _require_gpu(a, "a")
+    _require_gpu(b, "b")
+    assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0], f"shape mismatch {tuple(a.shape)} @ {tuple(b.shape)}"
+    assert a.dtype in _F8 and b.dtype in _F8, "operands must be float8_e4m3fn / float8_e5m2"
+    m, k = a.shape
+    n = b.shape[1]
+    unit = lambda t, d: t.shape[d] <= 1 or t.stride(d) == 1
+    a_rowmajor = unit(a, 1) and (m <= 1 or a.stride(0) >= k)   # [m][k] in memory
+    a_colmajor = unit(a, 0) and (k <= 1 or a.stride(1) >= m)   # [k][m] in memory
+    b_colmajor = unit(b, 0) and (n <= 1 or b.stride(1) >= k)   # [n][k] in memory: gemm_nt's bt
+    b_rowmajor = unit(b, 1) and (k <= 1 or b.stride(0) >= n)   # [k][n] in memory
+    if a_rowmajor and b_colmajor:
+        return gemm_nt(a, a_scale, b.t(), b_scale, out_dtype, bias=bias)
+    if b_rowmajor and (a_rowmajor or a_colmajor) and m > 0 and n > 0 and k > 1 and n > 1 and (a_rowmajor or m > 1):
+        for s in (a_scale, b_scale):
+            assert s.dtype == torch.float32 and s.numel() == 1 and s.device == a.device, "scales: 1 fp32 element on the operands' device"
+        if bias is not None:
+            assert bias.dtype == out_dtype and bias.numel() == n and bias.is_contiguous() and bias.device == a.device
+        _check_device(a.device)
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+        a_tr = not a_rowmajor
+        lda = a.stride(1) if a_tr else (a.stride(0) if m > 1 else k)
+        rc = lib().f8mi_gemm_ex(a.data_ptr(), _F8[a.dtype], int(a_tr), lda, b.data_ptr(), _F8[b.dtype], 1, b.stride(0), m, n, k,
+                                a_scale.data_ptr(), b_scale.data_ptr(), out.data_ptr(), _DT[out_dtype], n,
+                                bias.data_ptr() if bias is not None else None, _stream(a))
+        if rc == 0:
+            return out
+        if rc != ERR_UNSUPPORTED:
+            _check(rc, "f8mi_gemm_ex")
+    # the copies: gemm_nt makes an operand contiguous along k when it is not
+    return gemm_nt(a, a_scale, b.t(), b_scale, out_dtype, bias=bias)
 
 
 def sync_table(entries, device: torch.device) -> torch.Tensor:

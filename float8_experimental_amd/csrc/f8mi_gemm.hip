@@ -477,3 +477,35 @@ extern "C" int f8mi_gemm_kb_ex(const void* a, int a_fmt, int a_transposed, const
     return launch_gemm_dma16_nt(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, 64, m * 64, (const uint8_t*)bt, 64, k * 64, (int)m, (int)n,
                                 (int)k, scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
 }
+
+extern "C" int f8mi_gemm_ex(const void* a, int a_fmt, int a_transposed, int64_t lda, const void* bt, int b_fmt, int b_transposed, int64_t ldb,
+                            int64_t m, int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
+                            int64_t ldc, const void* bias_dev, void* stream_) {
+    if (!a_transposed && !b_transposed)
+        return f8mi_gemm_nt(a, a_fmt, lda, bt, b_fmt, ldb, m, n, k, scale_a_dev, scale_b_dev, c, c_dtype, ldc, bias_dev, stream_);
+    hipStream_t stream = (hipStream_t)stream_;
+    if (a_transposed && !b_transposed) { set_error("f8mi_gemm_ex: a transposed with bt not transposed is not built (copy a, or swap the operands and transpose c)"); return F8MI_ERR_UNSUPPORTED; }
+    if (m < 0 || n < 0 || k < 0 || ldc < n || lda < (a_transposed ? m : k) || ldb < n) { set_error("f8mi_gemm_ex: bad shape m=%lld n=%lld k=%lld lda=%lld ldb=%lld ldc=%lld", (long long)m, (long long)n, (long long)k, (long long)lda, (long long)ldb, (long long)ldc); return F8MI_ERR_INVALID_ARG; }
+    if (a_fmt < 0 || a_fmt > 1 || b_fmt < 0 || b_fmt > 1 || c_dtype < 0 || c_dtype > 2) { set_error("f8mi_gemm_ex: unknown format/dtype code"); return F8MI_ERR_INVALID_ARG; }
+    if (m == 0 || n == 0) return F8MI_OK;
+    if (!a || !bt || !c || !scale_a_dev || !scale_b_dev) { set_error("f8mi_gemm_ex: null pointer"); return F8MI_ERR_INVALID_ARG; }
+    // what the kernels that read an operand transposed need; anything else is for the caller to copy
+    if (k % 128 != 0 || k < 384) { set_error("f8mi_gemm_ex: transposed operands need k %% 128 == 0 and k >= 384 (k=%lld)", (long long)k); return F8MI_ERR_UNSUPPORTED; }
+    if (n % 64 != 0 || (a_transposed && m % 64 != 0)) { set_error("f8mi_gemm_ex: a transposed operand needs its row count to be a multiple of 64 (m=%lld n=%lld)", (long long)m, (long long)n); return F8MI_ERR_UNSUPPORTED; }
+    if ((uintptr_t)a % 16 != 0 || (uintptr_t)bt % 16 != 0 || lda % 16 != 0 || ldb % 16 != 0) { set_error("f8mi_gemm_ex: transposed operands need 16-byte aligned addresses and row strides"); return F8MI_ERR_UNSUPPORTED; }
+    if (((m + 127) / 128) * ((n + 127) / 128) <= 256) { set_error("f8mi_gemm_ex: an output of at most 256 tiles of 128 x 128 is faster from transposed copies (128-row tiles read no operand transposed)"); return F8MI_ERR_UNSUPPORTED; }
+    // 32-bit offsets inside a step: 128 contraction rows of a transposed operand, 256 rows of a normal one
+    if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff - BK || 128 * ldb + 256 > 0x7fffffffLL || (a_transposed ? 128 * lda + 256 : lda * (BM - 1) + k + BK) > 0x7fffffffLL) { set_error("f8mi_gemm_ex: dimension or row stride too large"); return F8MI_ERR_UNSUPPORTED; }
+    const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    if (tiles_m * tiles_n > 0x7fffffff) { set_error("f8mi_gemm_ex: too many tiles"); return F8MI_ERR_UNSUPPORTED; }
+    const int64_t csz = c_dtype == F8MI_FP32 ? 4 : 2;
+    const int c_vec_ok = (uintptr_t)c % csz == 0;
+    dim3 g((unsigned)(tiles_m * tiles_n));
+    ProfScope prof(F8MI_K_GEMM, 2.0 * (double)m * (double)n * (double)k, stream);
+    // a row-major matrix read transposed: row stride between contraction rows, 64 bytes between blocks of 64 rows
+    if (a_transposed)
+        return launch_gemm_dma16_tt(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, lda, 64, (const uint8_t*)bt, ldb, 64, (int)m, (int)n, (int)k,
+                                    scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+    return launch_gemm_dma16_nt(a_fmt, b_fmt, c_dtype, g, stream, (const uint8_t*)a, lda, 64, (const uint8_t*)bt, ldb, 64, (int)m, (int)n, (int)k,
+                                scale_a_dev, scale_b_dev, c, ldc, bias_dev, (int)tiles_m, (int)tiles_n, c_vec_ok);
+}

@@ -190,6 +190,9 @@ class Float8Linear(torch.nn.Linear):
 
     def __init__(self, *args, **kwargs):
         self.always_float32_buffers = set()  # before nn.Module.__init__: _apply may run early
+        # counts replacements of the delayed-scaling buffers (creation, .to(), ...): what caches of their addresses key on
+        self._buffer_gen = 0
+        self._static_marked_gen = -1
         config = kwargs.pop("config")
         super().__init__(*args, **kwargs)
         self.config = config
@@ -237,11 +240,22 @@ class Float8Linear(torch.nn.Linear):
     def register_always_float32_buffer(self, name: str, tensor: Optional[torch.Tensor], persistent: bool = True) -> None:
         self.register_buffer(name=name, tensor=tensor, persistent=persistent)
         self.always_float32_buffers.add(name)
+        self._buffer_gen += 1
 
     def _apply(self, fn, recurse=True):
         ret = super()._apply(fn, recurse)
         self.convert_amax_buffer_to_float32()
+        self._buffer_gen += 1
         return ret
+
+    def __setattr__(self, name, value):
+        if name in self.__dict__.get("always_float32_buffers", ()):  # a buffer assigned anew: addresses may have changed
+            self.__dict__["_buffer_gen"] = self.__dict__.get("_buffer_gen", 0) + 1
+        super().__setattr__(name, value)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)  # load_state_dict(assign=True) swaps the buffer tensors
+        self._buffer_gen += 1
 
     def convert_amax_buffer_to_float32(self):
         """``module.to(bf16)`` must not touch the bookkeeping precision (reference :224-238)."""

@@ -71,17 +71,29 @@ def get_float8_layers(model: torch.nn.Module) -> List[Float8Linear]:
     fp8_layers = [m for m in model.modules() if isinstance(m, Float8Linear)]
     if not torch.compiler.is_compiling():
         for layer in fp8_layers:
-            for buf in layer.buffers():
-                torch._dynamo.mark_static_address(buf, guard=True)
+            if layer._static_marked_gen != layer._buffer_gen:  # once per set of buffers, not on every call
+                for buf in layer.buffers():
+                    torch._dynamo.mark_static_address(buf, guard=True)
+                layer._static_marked_gen = layer._buffer_gen
     return fp8_layers
 
 
+_tables = {}
+
+
 def _sync_table(fp8_layers) -> torch.Tensor:
-    """Device table of (amax, history, scale, format) pointers for all 3L buffers (cached while the buffers stay
-    where they are)."""
-    return _native.sync_table_cached(
-        (getattr(child, f"fp8_amax_{kind}"), getattr(child, f"fp8_amax_history_{kind}"), getattr(child, f"fp8_scale_{kind}"), f8)
-        for child in fp8_layers for kind, f8 in _KINDS)
+    """Device table of (amax, history, scale, format) pointers for all 3L buffers.  Cached per list of layers for as
+    long as none of them has had its buffers replaced (``Float8Linear._buffer_gen`` counts that): a sync of 80 layers
+    then costs the host a tuple of 80 pairs instead of 720 pointer look-ups."""
+    key = tuple((id(child), child._buffer_gen) for child in fp8_layers)
+    hit = _tables.get(key)
+    if hit is None:
+        if len(_tables) > 16:
+            _tables.clear()
+        hit = _tables[key] = _native.sync_table_cached(
+            (getattr(child, f"fp8_amax_{kind}"), getattr(child, f"fp8_amax_history_{kind}"), getattr(child, f"fp8_scale_{kind}"), f8)
+            for child in fp8_layers for kind, f8 in _KINDS)
+    return hit
 
 
 @torch.no_grad()

@@ -13,7 +13,7 @@ from torch.utils._pytree import tree_map
 from . import float8_aten_api  # noqa: F401  (registers torch.ops.aten.mm_float8_emulated)
 from .float8_python_api import addmm_float8_unwrapped
 from .float8_tensor import choose_scaled_mm_config, Float8Tensor
-from .float8_utils import is_row_major, pad_tensor_for_matmul
+from .float8_utils import pad_tensor_for_matmul
 
 aten = torch.ops.aten
 FLOAT8_OPS_TABLE: Dict[Any, Any] = {}
@@ -83,19 +83,18 @@ def float8_cast_up_op(aten_op, args, kwargs=None):
 
 
 def preprocess_addmm(a: Float8Tensor, b: Float8Tensor):
-    """Operands of ``a @ b`` in the layout the kernel wants: ``a`` row-major, ``b`` column-major
-    (reference :131-155).  ``pad_inner_dim`` zero-pads the reduction to a multiple of 16 exactly
-    like the reference; zeros do not change the product and the kernel needs no padding."""
+    """Operands of ``a @ b`` for ``addmm_float8_unwrapped`` (reference :131-155).  ``pad_inner_dim`` zero-pads the
+    reduction to a multiple of 16 exactly like the reference; zeros do not change the product and the kernel needs
+    no padding.  The reference goes on to copy the payloads into the one layout ``torch._scaled_mm`` takes -- ``a``
+    row-major, ``b`` column-major (:150-153); here they are handed on as they lie: the kernel behind
+    ``addmm_float8_unwrapped`` reads a row-major ``b`` (and a column-major ``a``) transposed, and makes that copy
+    itself only for the small or ragged products where it cannot."""
     a_data, b_data = a._data, b._data
     cfg = choose_scaled_mm_config(a._gemm_input_role, a._linear_mm_config, b._gemm_input_role, b._linear_mm_config)
     if cfg.pad_inner_dim:
         assert a_data.size(1) == b_data.size(0), f"Inner dims must match for mm, got {a_data.size(1)} and {b_data.size(0)}"
         a_data = pad_tensor_for_matmul(a_data, dims=1)
         b_data = pad_tensor_for_matmul(b_data, dims=0)
-    if not is_row_major(a_data.stride()):
-        a_data = a_data.view(torch.uint8).contiguous().view(a_data.dtype)
-    if is_row_major(b_data.stride()):
-        b_data = b_data.view(torch.uint8).t().contiguous().t().view(b_data.dtype)
     return a_data, a._scale, b_data, b._scale
 
 

@@ -16,9 +16,11 @@ def addmm_float8_unwrapped(a_data: torch.Tensor, a_scale: torch.Tensor, b_data: 
 
     ``a_data`` is fp8 ``[m, k]``, ``b_data`` fp8 ``[k, n]``; as in the reference
     (float8_python_api.py:24-64) the scales are the tensors' forward scales and the
-    kernel applies their reciprocals.  The kernel wants both operands contiguous along
-    k: ``a_data`` row-major and ``b_data`` column-major pass through untouched (the
-    layout float8_ops.preprocess_addmm guarantees), anything else is copied once.
+    kernel applies their reciprocals.  Any layout is taken: ``a_data`` row-major with
+    ``b_data`` column-major (the pair ``torch._scaled_mm`` insists on) is read as it lies; a
+    row-major ``b_data`` -- and a column-major ``a_data`` next to it -- is read transposed by the
+    matrix-core kernel (f8mi_gemm_ex) where the product is large and aligned enough, and
+    copied once where it is not.
     ``use_fast_accum`` has no effect on this hardware.  ``output_scale`` (fp8 output) is
     not implemented, as in the reference's own call sites, which always pass None.
     """
@@ -26,4 +28,4 @@ def addmm_float8_unwrapped(a_data: torch.Tensor, a_scale: torch.Tensor, b_data: 
         raise NotImplementedError("fp8 output of the scaled matmul is not supported")
     assert a_data.dim() == 2 and b_data.dim() == 2 and a_data.shape[1] == b_data.shape[0]
     _native._require_gpu(a_data, "a_data")
-    return torch.ops.f8mi.gemm_nt(a_data, a_scale, b_data.t(), b_scale, output_dtype, bias)
+    return torch.ops.f8mi.scaled_mm(a_data, a_scale, b_data, b_scale, output_dtype, bias)

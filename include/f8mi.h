@@ -278,6 +278,22 @@ int f8mi_gemm_kb_ex(const void* a, int a_fmt, int a_transposed, const void* bt, 
                     int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
                     int64_t ldc, const void* bias_dev, void* stream);
 
+/* f8mi_gemm_nt on ROW-MAJOR fp8 operands either of which may be given transposed, so that the fp8 transposes
+ * preprocess_addmm makes for torch._scaled_mm's layout rule (a row-major, b column-major: float8_ops.py:131-155, the
+ * .t().contiguous().t() of :150-153) need not be made: the matrix-core kernel transposes on the way from LDS to the
+ * registers.
+ *   a, a_transposed = 0: [m][k], row stride lda >= k;  = 1: [k][m], row stride lda >= m (the memory of a.t())
+ *   bt, b_transposed = 0: [n][k], row stride ldb >= k; = 1: [k][n], row stride ldb >= n (b of a @ b, row-major)
+ * In the reference's words: forward x @ W.t() is (0, 0); grad_input dY @ W, W row-major, is (0, 1); grad_weight
+ * dY.t() @ x, both row-major, is (1, 1).  (0, 0) is f8mi_gemm_nt.  Transposed operands are taken when k % 128 == 0,
+ * k >= 384, the transposed operand's row count (n; m too for (1, 1)) is a multiple of 64, addresses and row strides
+ * are 16-byte aligned and the output has more than 256 tiles of 128 x 128; otherwise, and for (1, 0), the call
+ * returns F8MI_ERR_UNSUPPORTED without having launched anything and the caller makes the copy the reference makes.
+ * Same result bits as f8mi_gemm_nt on the copies. */
+int f8mi_gemm_ex(const void* a, int a_fmt, int a_transposed, int64_t lda, const void* bt, int b_fmt, int b_transposed, int64_t ldb,
+                 int64_t m, int64_t n, int64_t k, const float* scale_a_dev, const float* scale_b_dev, void* c, int c_dtype,
+                 int64_t ldc, const void* bias_dev, void* stream);
+
 /* One (layer, tensor) row of the delayed-scaling bookkeeping; all device pointers. */
 typedef struct f8mi_sync_entry {
     float* amax;    /* [1]        fp8_amax_*          */

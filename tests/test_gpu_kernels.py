@@ -806,6 +806,36 @@ def test_gemm_on_zero_padded_kblocked_operands(nat, m, n, k):
     _gemm_check(nat, m, n, k, "e5m2", "e4m3", torch.bfloat16, seed=m + n + k)
 
 
+@pytest.mark.parametrize("m,n,k", [(16, 128, 48), (16, 128, 41), (2048, 4096, 2048), (4096, 2048, 384), (2112, 2176, 640),
+                                   (2050, 4096, 1024), (4096, 2100, 1024), (16384, 8192, 8192)])
+def test_scaled_mm_on_row_major_operands_equals_the_copy_route_bitwise(nat, m, n, k):
+    """f8mi_gemm_ex / scaled_mm: a @ b with b row-major (the grad_input product) and with a column-major as well (the
+    grad_weight product) gives the bits of gemm_nt on the copies preprocess_addmm would have made -- read transposed by
+    the kernel where the product is large and aligned (checked through the return code), copied where it is not."""
+    a = _rand_fp8((m, k), torch.float8_e5m2, m + k, 4.0).to(DEV)
+    b = _rand_fp8((k, n), torch.float8_e4m3fn, n + k, 4.0).to(DEV)            # row-major [k, n]
+    a_cm = a.view(torch.uint8).t().contiguous().view(a.dtype).t()               # the same matrix, column-major
+    bt = b.view(torch.uint8).t().contiguous().view(b.dtype)                     # [n, k]: what gemm_nt takes
+    sa, sb = torch.tensor(3.0, device=DEV), torch.tensor(0.5, device=DEV)
+    bias = (torch.randn(n) * 3).to(torch.bfloat16).to(DEV)
+    for out_dt, bi in ((torch.bfloat16, bias), (torch.float32, None)):
+        want = nat.gemm_nt(a, sa, bt, sb, out_dt, bias=bi, split_k=False)
+        assert torch.equal(nat.scaled_mm(a, sa, b, sb, out_dt, bias=bi), want), (m, n, k, out_dt, "b row-major")
+        assert torch.equal(nat.scaled_mm(a_cm, sa, b, sb, out_dt, bias=bi), want), (m, n, k, out_dt, "a column-major, b row-major")
+        assert torch.equal(nat.scaled_mm(a, sa, bt.t(), sb, out_dt, bias=bi), want)
+        assert torch.equal(nat.scaled_mm(a_cm, sa, bt.t(), sb, out_dt, bias=bi), want)   # (1, 0): a is copied
+    # which of them the kernel took without a copy
+    L = nat.lib()
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    fast_b = k % 128 == 0 and k >= 384 and n % 64 == 0 and -(-m // 128) * -(-n // 128) > 256
+    rc = L.f8mi_gemm_ex(a.data_ptr(), 1, 0, k, b.data_ptr(), 0, 1, n, m, n, k, sa.data_ptr(), sb.data_ptr(), out.data_ptr(), 0, n, None, None)
+    assert rc == (0 if fast_b else nat.ERR_UNSUPPORTED), (m, n, k, rc)
+    rc = L.f8mi_gemm_ex(a_cm.data_ptr(), 1, 1, m, b.data_ptr(), 0, 1, n, m, n, k, sa.data_ptr(), sb.data_ptr(), out.data_ptr(), 0, n, None, None)
+    assert rc == (0 if fast_b and m % 64 == 0 else nat.ERR_UNSUPPORTED), (m, n, k, rc)
+    rc = L.f8mi_gemm_ex(a_cm.data_ptr(), 1, 1, m, bt.data_ptr(), 0, 0, k, m, n, k, sa.data_ptr(), sb.data_ptr(), out.data_ptr(), 0, n, None, None)
+    assert rc == nat.ERR_UNSUPPORTED
+
+
 def test_gemm_kblocked_refuses_short_or_ragged_k(nat):
     s1 = torch.ones((), device=DEV)
     for k in (64, 320):

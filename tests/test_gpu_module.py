@@ -467,6 +467,36 @@ def test_cfg1_against_the_reference_fixture(f8):
         assert abs(val.double().norm().item() / float(g[key]) - 1) < 1e-3, key
 
 
+def test_sync_follows_buffers_that_are_replaced(f8):
+    """sync keeps a table of buffer addresses per list of layers; every way of replacing a buffer tensor -- assignment,
+    .to(), load_state_dict(assign=True) -- makes it rebuild the table, so the scales always come from the buffers the
+    modules hold now."""
+    cfg = _cfg(f8, "del", "del", "del", hist=4)
+    model = nn.Sequential(*[f8.Float8Linear.from_float(nn.Linear(64, 64, bias=False), config=cfg) for _ in range(3)]).to(DEV)
+    for mod in model:
+        mod.last_seen_input_dtype = torch.bfloat16
+
+    def scales():
+        return [getattr(mod, f"fp8_scale_{kind}").item() for mod in model for kind in ("input", "weight", "grad_output")]
+
+    f8.sync_float8_amax_and_scale_history(model)
+    assert scales() == [1.0] * 9                     # default amax = fmax of the format
+    model[1].fp8_amax_weight = torch.tensor([7.0], device=DEV)          # a new tensor under the same name
+    f8.sync_float8_amax_and_scale_history(model)
+    assert scales()[4] == 448.0 * np.float32(1.0 / 7.0) and scales()[:4] == [1.0] * 4
+    model.to("cpu")
+    model.to(DEV)                                                       # every buffer moved
+    model[2].fp8_amax_grad_output.fill_(2.0)
+    f8.sync_float8_amax_and_scale_history(model)
+    assert scales()[8] == 57344.0 / 2.0 and scales()[4] == 448.0 * np.float32(1.0 / 7.0)
+    sd = {k: v.clone() for k, v in model.state_dict().items()}
+    sd["0.fp8_amax_input"] = torch.tensor([14.0], device=DEV)
+    model.load_state_dict(sd, assign=True)                              # every buffer swapped for the dict's tensor
+    f8.sync_float8_amax_and_scale_history(model)
+    assert scales()[0] == 448.0 * np.float32(1.0 / 14.0) and scales()[8] == 57344.0 / 2.0
+    assert model[0].fp8_scale_input.data_ptr() == sd["0.fp8_scale_input"].data_ptr()
+
+
 # --------------------------------------------------------------- config 5
 
 
