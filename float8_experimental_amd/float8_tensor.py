@@ -78,10 +78,17 @@ class _ToFloat8ConstrFunc(torch.autograd.Function):
     def forward(ctx, tensor, scale, float8_dtype=e4m3_dtype, linear_mm_config=None,
                 gemm_input_role=GemmInputRole.INPUT, amax_buffer=None):
         _native._require_gpu(tensor, "tensor")
-        # amax_buffer (delayed scaling): max|tensor| comes out of the same kernel and is copied there
-        bits, amax = torch.ops.f8mi.cast(tensor, scale, float8_dtype, _product_dtype(tensor, scale), amax_buffer is not None)
-        if amax_buffer is not None:
-            amax_buffer.copy_(amax.reshape(amax_buffer.shape))
+        plain = (torch.Tensor, torch.nn.Parameter)
+        if (amax_buffer is not None and not torch.compiler.is_compiling() and type(tensor) in plain
+                and type(amax_buffer) in plain and amax_buffer.dtype == torch.float32 and amax_buffer.numel() == 1):
+            # eager mode, delayed scaling: the kernel writes max|tensor| into the module's buffer itself (no
+            # temporary, no copy launch)
+            bits, _ = _native.cast(tensor, scale, float8_dtype, product_dtype=_product_dtype(tensor, scale), amax_out=amax_buffer)
+        else:
+            # one opaque node for torch.compile; functional, so the amax comes back and is copied into the buffer
+            bits, amax = torch.ops.f8mi.cast(tensor, scale, float8_dtype, _product_dtype(tensor, scale), amax_buffer is not None)
+            if amax_buffer is not None:
+                amax_buffer.copy_(amax.reshape(amax_buffer.shape))
         return Float8Tensor(bits, scale, tensor.dtype, linear_mm_config=linear_mm_config,
                             gemm_input_role=gemm_input_role)
 

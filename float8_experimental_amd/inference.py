@@ -62,25 +62,36 @@ class QuantConfig:
 
 
 def _to_kblock(rowmajor_fp8: torch.Tensor) -> torch.Tensor:
-    """[rows, k] fp8 bytes -> [k/64, rows, 64]: the placement f8mi_gemm_nt_kb reads (bytes moved, not changed)."""
+    """[rows, k] fp8 bytes -> [k/64, rows, 64]: the placement f8mi_gemm_nt_kb reads (bytes moved, not changed); a k that
+    is no multiple of 64 is extended with zero bytes to a multiple of 128 first (F8MI_LAYOUT_KBLOCK64_PAD128)."""
     rows, k = rowmajor_fp8.shape
     kb = _native.KB
-    return (rowmajor_fp8.view(torch.uint8).view(rows, k // kb, kb).permute(1, 0, 2).contiguous().view(rowmajor_fp8.dtype))
+    data = rowmajor_fp8.view(torch.uint8)
+    if k % kb != 0:
+        data = torch.nn.functional.pad(data, (0, _native.padded_k(k) - k))
+    return data.view(rows, data.shape[1] // kb, kb).permute(1, 0, 2).contiguous().view(rowmajor_fp8.dtype)
 
 
-# k-blocked copies of quantised weights, by the address of the row-major bytes; rebuilt when those bytes change
+# k-blocked copies of quantised weights, by the address of the row-major bytes; refreshed when those bytes change
 # (version counter) and dropped with the weight.  Module-level so that the custom op, which sees plain tensors, finds it.
 _KB_WEIGHTS = {}
 
 
 def _kblocked_weight(w_data: torch.Tensor) -> torch.Tensor:
+    """The k-blocked copy of a quantised weight.  An in-place update of the weight (``copy_``, ``load_state_dict``)
+    refreshes the copy IN PLACE: its address stays what a captured graph (``torch.compile(mode="reduce-overhead")``, a
+    HIP graph) recorded, so replays read the new bytes once any eager call has come by; only a weight of another shape
+    or dtype at the same address gets a new copy."""
     key = w_data.data_ptr()
-    tag = (w_data._version, tuple(w_data.shape), w_data.dtype)
+    tag = (tuple(w_data.shape), w_data.dtype)
     hit = _KB_WEIGHTS.get(key)
     if hit is None or hit[0] != tag:
         if hit is None:
             weakref.finalize(w_data, _KB_WEIGHTS.pop, key, None)
-        hit = _KB_WEIGHTS[key] = (tag, _to_kblock(w_data))
+        hit = _KB_WEIGHTS[key] = [tag, _to_kblock(w_data), w_data._version]
+    elif hit[2] != w_data._version:
+        hit[1].view(torch.uint8).copy_(_to_kblock(w_data).view(torch.uint8))
+        hit[2] = w_data._version
     return hit[1]
 
 
@@ -89,7 +100,7 @@ def _fp8_linear(x2: torch.Tensor, w_data: torch.Tensor, w_scale: torch.Tensor, s
     """x2 [m, k] high precision, w_data [n, k] fp8 row-major -> [m, n] in x2's dtype: activation cast (static scale if
     given, else dynamic) and the scaled GEMM with the bias in its epilogue."""
     k = x2.shape[1]
-    use_kb = _native.kblock_ok(k)
+    use_kb = _native.kblock_layout(k)  # row-major for a short contraction, else k-blocked (zero-padded when ragged)
     if static_scale is not None:
         scale = static_scale
         x8, _ = _native.cast(x2, scale, e4m3_dtype, product_dtype=_product_dtype(x2, scale), out_kblock=use_kb)
@@ -167,7 +178,7 @@ class Float8InferenceLinear(torch.nn.Linear):
                                                          GemmInputRole.WEIGHT)
         self.weight = nn.Parameter(quantized_weight)
         self.weight.requires_grad = False
-        if quantized_weight._data.is_cuda and _native.kblock_ok(self.in_features):
+        if quantized_weight._data.is_cuda and _native.kblock_layout(self.in_features) != _native.ROWMAJOR:
             self._weight_kblocked()  # now, not inside the first forward (which may be a node of a compiled graph)
 
     def set_weight_and_bias(self, weight: torch.nn.Parameter, bias: Optional[torch.nn.Parameter]):

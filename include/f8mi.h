@@ -220,7 +220,12 @@ int f8mi_cast_dynamic(const void* x, int64_t rows, int64_t cols, int64_t ld, int
  * same result bits as f8mi_cast_dynamic.  All calls on one GPU share the one array: calls that can overlap in time
  * on the same GPU (two streams, two host threads) race on it -- give such callers f8mi_cast_dynamic and a workspace
  * each.  The array keeps the last call's contents; nothing in it needs to start at zero.  Tensors of more than
- * F8MI_STATIC_MAX_ELEMS elements are refused with F8MI_ERR_INVALID_ARG. */
+ * F8MI_STATIC_MAX_ELEMS elements are refused with F8MI_ERR_INVALID_ARG.
+ * The first call on a device asks the runtime for the array's address on the device that is current (which, as for
+ * every entry point, must be the device `stream` belongs to); that query may load the library's code onto the device
+ * and is not something to do while a stream is being captured.  Make one ordinary call on each device before the
+ * first capture (any size will do); from then on the entry point only launches kernels and may be captured and
+ * replayed. */
 #define F8MI_STATIC_SCRATCH_BYTES 4096
 #define F8MI_STATIC_MAX_ELEMS (1ll << 36)
 int f8mi_cast_dynamic_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_dtype, int fp8_fmt,

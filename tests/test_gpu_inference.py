@@ -102,7 +102,8 @@ def test_mlp_flows_compile_fullgraph(f8, backend, dtype, mode):
         assert _sqnr(f8, eager, got) > 25 and _sqnr(f8, eager2, got2) > 25
 
 
-@pytest.mark.parametrize("shape,bias", [((3, 40, 512), True), ((130, 448), False), ((7, 200), True), ((64, 4096), True)])
+@pytest.mark.parametrize("shape,bias", [((3, 40, 512), True), ((130, 448), False), ((7, 200), True), ((64, 4096), True),
+                                        ((300, 1000), True), ((20, 4097), False)])
 @pytest.mark.parametrize("static", [False, True])
 def test_fast_path_equals_the_composed_float8tensor_route_and_the_oracle(f8, shape, bias, static):
     """The module's own route (cast in the GEMM's layout, bias in the epilogue) against the reference's
@@ -136,6 +137,43 @@ def test_fast_path_equals_the_composed_float8tensor_route_and_the_oracle(f8, sha
         want = want + lin.bias.detach().float()
     err = (got.float().cpu().reshape(-1, n) - want).abs().max().item() / want.abs().max().item()
     assert err <= 1e-2, err
+
+
+def test_in_place_weight_update_reaches_eager_and_captured_calls(f8):
+    """The module keeps a k-blocked copy of the quantised weight for the GEMM.  Overwriting the weight's bytes in place
+    (what load_state_dict does) must show in the next eager call AND in replays of a HIP graph captured before the
+    update: the copy is refreshed in place, at the address the graph recorded, by the first eager call after it."""
+    from float8_experimental_amd.inference import ActivationCasting, Float8InferenceLinear, QuantConfig
+
+    torch.manual_seed(3)
+    k, n = 1024, 768
+    lin_a, lin_b = nn.Linear(k, n, bias=False).to(torch.bfloat16).to(DEV), nn.Linear(k, n, bias=False).to(torch.bfloat16).to(DEV)
+    cfg = QuantConfig(ActivationCasting.DYNAMIC)
+    mod = Float8InferenceLinear.from_float(copy.deepcopy(lin_a), cfg, use_fast_accum=True)
+    other = Float8InferenceLinear.from_float(copy.deepcopy(lin_b), cfg, use_fast_accum=True)
+    x = (torch.randn(256, k, device=DEV) * 2).to(torch.bfloat16)
+    y_static = torch.empty(256, n, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        want_a, want_b = mod(x), other(x)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            mod(x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static.copy_(mod(x))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_static, want_a)
+        before = mod._weight_kblocked().data_ptr()
+        mod.weight._data.view(torch.uint8).copy_(other.weight._data.view(torch.uint8))   # in place: same storage, new version
+        mod.weight._scale.copy_(other.weight._scale)
+        assert torch.equal(mod(x), want_b)                     # eager sees the new bytes
+        assert mod._weight_kblocked().data_ptr() == before     # ... in the same k-blocked buffer
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_static, want_b)                   # and so does the graph captured before the update
 
 
 def test_weight_only_dequantises_and_ignores_the_bias_like_the_reference(f8):

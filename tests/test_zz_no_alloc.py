@@ -85,3 +85,44 @@ def test_static_entry_point_refuses_what_it_cannot_take(native):
     assert rc == -1 and b"at most" in lib.f8mi_last_error()
     rc = lib.f8mi_cast_dynamic_static(C.c_void_p(16), i64(4), i64(4), i64(4), 0, 0, None, C.c_void_p(16), 0, None, 0, None)
     assert rc == -1 and b"scale" in lib.f8mi_last_error()
+
+
+def test_static_entry_point_captured_in_a_graph_and_replayed(native):
+    """The use the entry point is for: captured into a HIP graph (after one ordinary call on the device, which looks
+    the array's address up) and replayed on new contents of the same input buffer -- every replay against
+    f8mi_cast_dynamic on the same contents, with eager work and synchronisation between the replays."""
+    lib = native.lib()
+    torch.manual_seed(7)
+    rows, cols = 1024, 2048
+    x = torch.randn(rows, cols, device=DEV).to(torch.bfloat16)
+    scale = torch.zeros(1, dtype=torch.float32, device=DEV)
+    out = torch.zeros(rows * cols, dtype=torch.uint8, device=DEV)
+    out_t = torch.zeros(rows * cols, dtype=torch.uint8, device=DEV)
+    ws = torch.zeros(lib.f8mi_workspace_bytes() // 4, dtype=torch.int32, device=DEV)
+
+    def static_call(stream):
+        rc = lib.f8mi_cast_dynamic_static(x.data_ptr(), rows, cols, cols, 0, 0, scale.data_ptr(), out.data_ptr(), 1, out_t.data_ptr(), 1, stream)
+        assert rc == 0, lib.f8mi_last_error()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        static_call(side.cuda_stream)            # the warm-up call, outside any capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call(torch.cuda.current_stream().cuda_stream)
+    for i in range(4):
+        x.copy_((torch.randn(rows, cols, device=DEV) * (0.01 * 10.0 ** i)).to(torch.bfloat16))   # eager work between replays
+        out.zero_()
+        out_t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        s_ref = torch.zeros(1, dtype=torch.float32, device=DEV)
+        o_ref, t_ref = torch.zeros_like(out), torch.zeros_like(out_t)
+        rc = lib.f8mi_cast_dynamic(x.data_ptr(), rows, cols, cols, 0, 0, s_ref.data_ptr(), o_ref.data_ptr(), 1, t_ref.data_ptr(), 1,
+                                   ws.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        assert scale.item() == s_ref.item(), (i, scale.item(), s_ref.item())
+        assert torch.equal(out, o_ref) and torch.equal(out_t, t_ref), i
