@@ -151,6 +151,10 @@ def parse():
     p.add_argument("--mfma-order", type=int, default=0, choices=[0, 1, 2, 3],
                    help="register-only MFMA loop: which operand changes between consecutive instructions "
                         "(0 the first, as in the GEMM; 1 the second; 2 both; 3 neither for eight in a row)")
+    p.add_argument("--per-gemm-only", type=float, default=None, metavar="SECONDS",
+                   help="run nothing but the twelve products of a step, each alone, through this library and through "
+                        "torch._scaled_mm (for profiler runs that compare the two kernels product by product); SECONDS > 0 "
+                        "also loops each for that long and samples socket power and shader clock")
     p.add_argument("--no-other-configs", action="store_true",
                    help="leave out the configurations besides the headline one (profiler runs of the headline's kernels)")
     p.add_argument("--calibrate-copy", action="store_true",
@@ -242,11 +246,13 @@ def probe_mfma(torch, random_data, iters=4000, operands=None, seconds=0.8, order
     return out
 
 
-def vendor_scaled_mm(torch, _native, layers, m, flop_step, iters):
+def vendor_scaled_mm(torch, _native, layers, m, flop_step, iters, seconds=0.0):
     """The same twelve products through torch._scaled_mm (hipBLASLt) on row-major fp8 operands with the transposed
     copies it needs made beforehand -- a reference point for the GEMM kernel, outside the timed region: all twelve back
     to back, and each product alone against this library's kernel on the same bytes (one fp8 copy per tensor, read as
-    it lies or transposed).  An "error" entry where the installed torch refuses a product (format pair or layout)."""
+    it lies or transposed).  ``seconds`` > 0: each product is also looped for that long per kernel with the socket
+    power and shader clock sampled over the second half (what rate, power and clock each settles at).  An "error" entry
+    where the installed torch refuses a product (format pair or layout)."""
     E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
     bf16 = torch.bfloat16
     rowmajor = lambda t: t.permute(1, 0, 2).reshape(t.shape[1], -1).contiguous()
@@ -260,6 +266,24 @@ def vendor_scaled_mm(torch, _native, layers, m, flop_step, iters):
             fn()
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / n
+
+    def settled(fn, flop):
+        t_end = time.perf_counter() + seconds / 2
+        while time.perf_counter() < t_end:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+        tele = Telemetry()
+        tele.start()
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds / 2:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+            n += 10
+        dt = (time.perf_counter() - t0) / n
+        t = tele.stop() or {}
+        return {"TFLOP/s": flop / dt / 1e12, "socket_power_W": t.get("socket_power_W_mean"), "sclk_MHz": t.get("sclk_MHz_mean")}
 
     try:
         per_gemm, vendor_all, ours_all = [], [], []
@@ -281,8 +305,12 @@ def vendor_scaled_mm(torch, _native, layers, m, flop_step, iters):
             flop = 2.0 * m * k * n
             for what, ours, theirs in products:
                 t_ours, t_theirs = timed_loop(ours, iters), timed_loop(theirs, iters)
-                per_gemm.append({"shape": name, "product": what, "this_library_TFLOP/s": flop / t_ours / 1e12,
-                                 "scaled_mm_TFLOP/s": flop / t_theirs / 1e12})
+                row = {"shape": name, "product": what, "this_library_TFLOP/s": flop / t_ours / 1e12,
+                       "scaled_mm_TFLOP/s": flop / t_theirs / 1e12}
+                if seconds > 0:
+                    row["this_library_settled"] = settled(ours, flop)
+                    row["scaled_mm_settled"] = settled(theirs, flop)
+                per_gemm.append(row)
                 vendor_all.append(t_theirs)
                 ours_all.append(t_ours)
             del x8, w8, g8, x8r, w8r, g8r, w8t, g8t, x8t, products
@@ -504,6 +532,11 @@ def main():
     idle.start()
     time.sleep(0.3)
     idle_w = (idle.stop() or {}).get("socket_power_W_mean")
+
+    if args.per_gemm_only is not None:
+        print(json.dumps({"per_gemm_only": vendor_scaled_mm(torch, _native, layers, m, flop_step, max(2, args.steps), args.per_gemm_only),
+                          "library_build_knobs": _native.build_knobs()}))
+        return
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
