@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define F8MI_VERSION 100
+#define F8MI_VERSION 110
 
 #define F8MI_OK 0
 #define F8MI_ERR_INVALID_ARG (-1) /* null pointer, negative size, unknown enum            */
