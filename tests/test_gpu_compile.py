@@ -64,9 +64,10 @@ def _run(mod, x, dy):
 
 @pytest.mark.parametrize("backend", ["eager", "aot_eager"])
 @pytest.mark.parametrize("bias", [False, True])
-@pytest.mark.parametrize("shape,n", [((4, 96, 512), 448), ((130, 200), 448), ((3, 768, 2048), 2432)])
+@pytest.mark.parametrize("shape,n", [((4, 96, 512), 448), ((130, 200), 448), ((3, 768, 2048), 2432), ((5, 83, 1000), 523)])
 def test_dynamic_scaling_compiles_as_one_graph(f8, backend, bias, shape, n):
-    # the last case's first layer is large enough for one fp8 copy per tensor, read transposed in backward
+    # the third case's first layer is large enough for one fp8 copy per tensor, read transposed in backward; the last
+    # case is ragged in every dimension: zero-padded k-blocked copies, whose shapes the fake implementations must predict
     torch.manual_seed(0)
     k = shape[-1]
     model = nn.Sequential(nn.Linear(k, n, bias=bias), nn.ReLU(), nn.Linear(n, 384, bias=bias)).to(DEV, dtype=torch.bfloat16)
@@ -105,7 +106,7 @@ def test_frozen_weight_and_no_grad_under_compile(f8):
 
 @pytest.mark.parametrize("backend", ["eager", "aot_eager"])
 @pytest.mark.parametrize("kinds", ["DDD", "DyD", "yDy"])  # input, weight, grad_output: D delayed, y dynamic
-@pytest.mark.parametrize("shape,n", [((32, 512), 448), ((3, 768, 2048), 2432)])
+@pytest.mark.parametrize("shape,n", [((32, 512), 448), ((3, 768, 2048), 2432), ((5, 83, 1000), 523)])
 def test_delayed_scaling_compiles_as_one_graph(f8, backend, kinds, shape, n):
     """Reference: test_compile.py runs delayed scaling with enable_amax_init=False, enable_pre_and_post_forward=False
     under fullgraph=True.  Here the amax buffers are written by the graph; the sync stays an eager call between steps."""

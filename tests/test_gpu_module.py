@@ -537,6 +537,47 @@ def test_cfg5_ragged_heavy_tailed(f8, m, k, n):
     _gemm_close(mod.weight.grad, ref["dw"], 1e-2, "dw")
 
 
+def test_ragged_layers_random_sweep_against_the_oracle(f8):
+    """Thirty layers with sizes that are multiples of nothing (and a few that are), dynamic and delayed scaling: every
+    contraction that reaches 384 once padded runs on zero-padded k-blocked copies.  Scales and amax buffers bit-exact,
+    y / dx / dw within 1e-2 of the emulated oracle."""
+    from oracle import torch_oracle as to
+
+    g = torch.Generator().manual_seed(2024)
+    pick = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    for case in range(30):
+        m, k, n = pick(1, 1400), pick(1, 1400), pick(1, 1400)
+        if case % 5 == 0:
+            m, k, n = 64 * pick(1, 12), 64 * pick(1, 12), 64 * pick(1, 12)
+        delayed = case % 3 == 2
+        x = (torch.randn(m, k, generator=g) * 3).to(torch.bfloat16)
+        w = (torch.randn(n, k, generator=g) * 0.2).to(torch.bfloat16)
+        dy = (torch.randn(m, n, generator=g) * 0.05).to(torch.bfloat16)
+        lin = nn.Linear(k, n, bias=False).to(torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.copy_(w)
+        mod = f8.Float8Linear.from_float(lin, config=_cfg(f8, *(("del",) * 3 if delayed else ("dyn",) * 3))).to(DEV)
+        xd = x.to(DEV).requires_grad_()
+        y = mod(xd)
+        y.backward(dy.to(DEV))
+        if delayed:
+            # first iteration: the scales come from this step's amaxes (amax init), in fp32
+            amax = lambda t: t.abs().max().float()
+            for kind, t, fmax in (("input", x, 448.0), ("weight", w, 448.0), ("grad_output", dy, 57344.0)):
+                assert getattr(mod, f"fp8_amax_{kind}").item() == amax(t).item(), (case, kind)
+                want = np.float32(fmax) * (np.float32(1.0) / np.float32(max(amax(t).item(), 1e-12)))
+                assert getattr(mod, f"fp8_scale_{kind}").item() == want, (case, kind)
+            sx, sw, sg = (getattr(mod, f"fp8_scale_{kind}").cpu() for kind in ("input", "weight", "grad_output"))
+            x8, w8, g8 = to.cast_to_fp8(x, sx, torch.float8_e4m3fn), to.cast_to_fp8(w, sw, torch.float8_e4m3fn), to.cast_to_fp8(dy, sg, torch.float8_e5m2)
+            ref = {"y": to.mm_emulated(x8, sx, w8.t(), sw, torch.bfloat16), "dx": to.mm_emulated(g8, sg, w8, sw, torch.bfloat16),
+                   "dw": to.mm_emulated(g8.t(), sg, x8, sx, torch.bfloat16)}
+        else:
+            ref = to.linear_fwd_bwd_dynamic(x, w, dy)
+        _gemm_close(y, ref["y"], 1e-2, ("y", case, m, k, n))
+        _gemm_close(xd.grad, ref["dx"], 1e-2, ("dx", case, m, k, n))
+        _gemm_close(mod.weight.grad, ref["dw"], 1e-2, ("dw", case, m, k, n))
+
+
 # ------------------------------------------------- LLaMa FFN integration
 
 
