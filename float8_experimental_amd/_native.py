@@ -236,7 +236,11 @@ def delayed_workspace(dev: torch.device) -> torch.Tensor:
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), _raw_stream(dev))
     ws = _delayed_workspaces.get(key)
     if ws is None:
-        ws = _delayed_workspaces[key] = torch.zeros(words, dtype=torch.int32, device=dev)
+        ws = torch.zeros(words, dtype=torch.int32, device=dev)
+        # under stream capture the fill is recorded, not run: such a tensor is zero only inside replays of that graph,
+        # so it serves this call and is not kept for later, eager calls on a stream with the same handle
+        if not torch.cuda.is_current_stream_capturing():
+            _delayed_workspaces[key] = ws
     return ws
 
 

@@ -1,5 +1,6 @@
 """Module swap and delayed-scaling bookkeeping (mirror of the reference's ``float8_linear_utils.py``)."""
 import logging
+import weakref
 from typing import Callable, List, Optional
 
 import torch
@@ -84,16 +85,23 @@ _tables = {}
 def _sync_table(fp8_layers) -> torch.Tensor:
     """Device table of (amax, history, scale, format) pointers for all 3L buffers.  Cached per list of layers for as
     long as none of them has had its buffers replaced (``Float8Linear._buffer_gen`` counts that): a sync of 80 layers
-    then costs the host a tuple of 80 pairs instead of 720 pointer look-ups."""
+    then costs the host a tuple of 80 pairs and 80 weak-reference checks instead of 720 pointer look-ups.
+
+    ``id()`` of a layer that has been freed can come back for a new layer with the same generation count, so an
+    entry also keeps a weak reference to each layer and counts as a hit only while all of them are the layers asked
+    for; and it holds the buffer tensors themselves, so the addresses in the table stay allocated for as long as
+    the entry lives."""
     key = tuple((id(child), child._buffer_gen) for child in fp8_layers)
     hit = _tables.get(key)
-    if hit is None:
-        if len(_tables) > 16:
-            _tables.clear()
-        hit = _tables[key] = _native.sync_table_cached(
-            (getattr(child, f"fp8_amax_{kind}"), getattr(child, f"fp8_amax_history_{kind}"), getattr(child, f"fp8_scale_{kind}"), f8)
-            for child in fp8_layers for kind, f8 in _KINDS)
-    return hit
+    if hit is not None and all(ref() is child for ref, child in zip(hit[1], fp8_layers)):
+        return hit[0]
+    if len(_tables) > 16:
+        _tables.clear()
+    entries = [(getattr(child, f"fp8_amax_{kind}"), getattr(child, f"fp8_amax_history_{kind}"), getattr(child, f"fp8_scale_{kind}"), f8)
+               for child in fp8_layers for kind, f8 in _KINDS]
+    table = _native.sync_table_cached(entries)
+    _tables[key] = (table, [weakref.ref(child) for child in fp8_layers], entries)
+    return table
 
 
 @torch.no_grad()

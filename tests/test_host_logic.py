@@ -293,3 +293,41 @@ def test_get_float8_layers_marks_buffers_static():
         assert len(bufs) == 9
         for buf in bufs:
             assert getattr(buf, "_dynamo_static_input_type", None) == "guarded"
+
+
+def test_sync_table_cache_does_not_trust_a_recycled_object_id(monkeypatch):
+    """The pointer table of sync_float8_amax_and_scale_history is cached per (id(layer), buffer generation).  A layer
+    that has been freed can hand its id() to a new layer with the same generation count: an entry left by the dead
+    layer must not be served for the new one (it holds the dead layer's addresses)."""
+    import gc
+    import weakref
+
+    from float8_experimental_amd import float8_linear_utils as flu
+
+    cfg = f8.Float8LinearConfig(cast_config_input=f8.CastConfig(f8.ScalingType.DELAYED))
+    layer = Float8Linear.from_float(nn.Linear(8, 8), config=cfg)
+    built = []
+    monkeypatch.setattr(_native, "sync_table_cached", lambda entries: built.append(list(entries)) or ("table", len(built)))
+    monkeypatch.setattr(flu, "_tables", {})
+
+    first = flu._sync_table([layer])
+    assert flu._sync_table([layer]) is first and len(built) == 1  # same live layer, same buffers: a hit
+    assert [t for row in flu._tables[next(iter(flu._tables))][2] for t in row[:3]] == [
+        getattr(layer, f"fp8_{what}_{kind}") for kind in ("input", "weight", "grad_output") for what in ("amax", "amax_history", "scale")]
+
+    # what a dead layer of the same id and generation leaves behind
+    ghost = Float8Linear.from_float(nn.Linear(8, 8), config=cfg)
+    dead = weakref.ref(ghost)
+    del ghost
+    gc.collect()
+    assert dead() is None
+    key = ((id(layer), layer._buffer_gen),)
+    flu._tables[key] = ("stale", [dead], [])
+    fresh = flu._sync_table([layer])
+    assert fresh != "stale" and len(built) == 2
+    assert flu._sync_table([layer]) is fresh and len(built) == 2
+
+    # replaced buffers: the generation moves and the table is rebuilt from the new tensors
+    layer.fp8_amax_input = torch.zeros(())
+    assert flu._sync_table([layer]) is not fresh and len(built) == 3
+    assert built[-1][0][0] is layer.fp8_amax_input
