@@ -36,7 +36,7 @@ def listings(tmp_path_factory):
 @pytest.mark.parametrize("unit", UNITS)
 def test_accumulator_reads_keep_their_distance_from_the_mfma_that_writes_them(listings, unit):
     lines = listings[unit]
-    ends = [i for i, l in enumerate(lines) if "s_endpgm" in l]
+    ends = [i for i, l in enumerate(lines) if re.match(r"\.Lfunc_end\d+:", l)]  # one per kernel (a kernel may hold several s_endpgm)
     assert len(ends) >= 12, "expected one kernel per operand format pair, output type and parity of the step count"
     start = 0
     for end in ends:
