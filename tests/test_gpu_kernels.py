@@ -898,6 +898,28 @@ def test_gemm_strided_operands(nat):
         assert bool(((out.double() - want).abs() <= 2.0**-13 * bound).all())
 
 
+@pytest.mark.parametrize("out_dt", [torch.bfloat16, torch.float16])
+def test_gemm_epilogue_of_tiles_inside_c_equals_the_checked_one_bitwise(nat, out_dt):
+    """A 256 x 256 tile that lies inside C is written without bounds checks, one on the edge of C with them.  Dropping
+    the last 8 rows and columns of a product turns its last row and column of tiles from the first kind into the
+    second; what both products share must not change by a bit."""
+    m, n, k = 4096, 4096, 512
+    assert nat.gemm_plan(m, n, k)[0] == "tiles256" and nat.gemm_plan(m - 8, n - 8, k)[0] == "tiles256"
+    a = _rand_fp8((m, k), torch.float8_e5m2, 31).to(DEV)
+    bt = _rand_fp8((n, k), torch.float8_e4m3fn, 32).to(DEV)
+    sa, sb = torch.tensor(3.0, device=DEV), torch.tensor(0.37, device=DEV)
+    bias = torch.linspace(-1, 1, n).to(out_dt).to(DEV)
+    for b in (None, bias):
+        whole = nat.gemm_nt(a, sa, bt, sb, out_dt, bias=b)
+        part = nat.gemm_nt(a[:m - 8], sa, bt[:n - 8], sb, out_dt, bias=None if b is None else b[:n - 8].contiguous())
+        assert torch.equal(whole[:m - 8, :n - 8], part)
+        # and the tiles inside C against the exact product
+        exact = (a[:512].cpu().double() @ bt[:512].cpu().double().t()) / (3.0 * 0.37) + (0 if b is None else b[:512].cpu().double())
+        err = (whole[:512, :512].cpu().double() - exact).abs()
+        assert bool((err <= {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[out_dt] * exact.abs() + 2.0**-12 * (
+            a[:512].cpu().double().abs() @ bt[:512].cpu().double().abs().t()) / (3.0 * 0.37)).all())
+
+
 # ------------------------------------------------------------------ K4 sync
 
 
